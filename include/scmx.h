@@ -1,0 +1,174 @@
+/* scmx — C ABI of the MI355X (gfx950) SC-MXFP4 W4A8 linear-layer engine.
+ *
+ * Every entry point enqueues HIP kernels on the caller's stream and returns at once (stream-ordered, no implicit
+ * synchronisation).  Pointers are DEVICE pointers unless stated otherwise; the library never allocates or frees
+ * device memory and keeps no state between calls, so it is reentrant.  Return value: 0 on success, a negative
+ * SCMX_ERR_* code otherwise, with a message available from scmx_last_error() (thread-local).
+ *
+ * Each declaration names the function of the reference (shinyoungkang1/mxfp4-int8-m5) it replaces, as file:line.
+ * `T` tensors are bfloat16 (uint16_t bit patterns) — the model dtype the reference runs with.
+ *
+ * Weight storage (e2e/sc_format.py:4-15): per row n of an [N, K] matrix
+ *   codes   uint32 [N*K/8]   8 four-bit codes per word, element k = 8j+i in bits 4i..4i+3; code = sign<<3 | idx
+ *   bcodes  uint8  [N, K*bc_bits/(8*block)]  block b in bits bc_bits*(b % per_byte) of byte b / per_byte
+ *   wscale  float  [N]
+ * decoding to the INT8 operand q[n,k] = +-code_mag[idx] * mult[bcode[n, k/block]], W = wscale[n] * q.
+ */
+#ifndef SCMX_H
+#define SCMX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SCMX_OK 0
+#define SCMX_ERR_ARG (-1)      /* bad shape, null pointer, misaligned pointer */
+#define SCMX_ERR_FORMAT (-2)   /* weight format outside what the kernels decode */
+#define SCMX_ERR_LAUNCH (-3)   /* HIP reported an error at launch */
+#define SCMX_ERR_WORKSPACE (-4)/* caller-provided workspace too small */
+
+/* Epilogues of the GEMM / GEMV (e2e/sc_kernels.py:73-78, e2e/sc_moe.py:10). */
+#define SCMX_EPI_I32 0     /* INT32 accumulators */
+#define SCMX_EPI_SCALE 1   /* T(acc * xscale[m] * wscale[n]) */
+#define SCMX_EPI_RES 2     /* T(res + T(acc * xscale[m] * wscale[n])) */
+#define SCMX_EPI_SWIGLU 3  /* rows interleaved g,g,u,u: swiglu(T(g), T(u)) -> [M, N/2] */
+
+/* Weight format descriptor: the fields of sc_format.Format (e2e/sc_format.py:26-37), passed per call instead of
+ * the reference's process-global F.DEFAULT (e2e/sc_kernels.py:471-473). */
+typedef struct scmx_format {
+    int32_t block;        /* weights per block along K: 8, 16, 32, 64 or 128 */
+    int32_t bc_bits;      /* bits per block code: 1, 2, 4 or 8 */
+    int32_t n_mult;       /* entries used in mult[], <= 16 and <= 2^bc_bits */
+    int32_t code_mag[8];  /* magnitude of code index 0..7; max(code_mag) * max(mult) <= 127 */
+    int32_t mult[16];     /* integer block multipliers */
+} scmx_format;
+
+const char* scmx_version(void);
+const char* scmx_last_error(void);
+
+/* Fill `f` with the published SC-MXFP4 format: block 32, magnitudes 2 x E2M1, multipliers 1,2,4,8, 2-bit codes
+ * (sc_format.DEFAULT, e2e/sc_format.py:63). */
+void scmx_default_format(scmx_format* f);
+
+/* ---- dense prefill ------------------------------------------------------------------------------------------ */
+
+/* Packed weights -> INT8 [n_rows, K].  Replaces unpack_i8, e2e/sc_kernels.py:34-50,480-483 (and unpack_experts,
+ * e2e/sc_moe.py:203-206, with n_rows = E*N). */
+int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t* bcodes, int8_t* wq,
+                   int64_t n_rows, int64_t K, void* stream);
+
+/* Per-token symmetric INT8 of x T[M, K]: xq int8 [Mp, K], xs float [Mp]; rows >= M are zero with scale 0.
+ * Replaces act_quant, e2e/sc_kernels.py:200-229,554-563. */
+int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream);
+
+/* INT8 [M,K] x INT8 [N,K]^T -> INT32 [M,N] on INT8 MFMA.  Replaces mm_i8_i32, e2e/sc_kernels.py:53-71,486-495. */
+int scmx_mm_i8_i32(const int8_t* xq, const int8_t* wq, int32_t* acc, int M, int N, int K, void* stream);
+
+/* The same GEMM with the scaling epilogue applied in registers; `res` T[M,N] is read by SCMX_EPI_RES only.
+ * out: T[M,N] (epi 1,2), T[M,N/2] (epi 3).  Replaces mm_epi, e2e/sc_kernels.py:79-115,498-508. */
+int scmx_mm_epi(const int8_t* xq, const int8_t* wq, const float* xscale, const float* wscale, const uint16_t* res,
+                void* out, int epi, int M, int N, int K, void* stream);
+
+/* mm_epi reading the PACKED weights: each workgroup unpacks its weight tile into LDS as exact INT8 and feeds the
+ * INT8 MFMA from there, so no INT8 copy of the weights is ever written (the in-kernel unpack of
+ * e2e/sc_moe.py:42-69 applied to the dense path; replaces the unpack_i8 + mm_epi pair of
+ * e2e/fused_qwen3.py:161-172).  epi 0 writes INT32 [M,N]. */
+int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, const uint32_t* codes,
+                 const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M, int N,
+                 int K, void* stream);
+
+/* Whole dense W4A8 linear on a bf16 input: activation quantization prologue + scmx_mm_w4a8, one call.
+ * workspace must hold scmx_linear_w4a8_workspace(M, K) bytes (the INT8 activations and their scales). */
+size_t scmx_linear_w4a8_workspace(int M, int K);
+int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* codes, const uint8_t* bcodes,
+                     const float* wscale, const uint16_t* res, void* out, int epi, int M, int N, int K,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- row kernels of the model integrations -------------------------------------------------------------------- */
+
+/* RMSNorm(x, w, eps) then per-token INT8; xn (optional, may be NULL) receives the normalized T rows [Mp, K].
+ * Replaces rmsnorm_quant / rmsnorm_quant_n, e2e/sc_kernels.py:123-174,383-386,527-533,619-626. */
+int scmx_rmsnorm_quant(const uint16_t* x, const uint16_t* w, float eps, int8_t* xq, float* xs, uint16_t* xn, int M,
+                       int Mp, int K, void* stream);
+
+/* h = res + T(acc*xscale*wscale) written to h; then, when xq != NULL, RMSNorm(h, w, eps) + INT8.
+ * Replaces res_norm_quant (e2e/sc_kernels.py:177-189,536-544) and res_epilogue (:191-197,547-551). */
+int scmx_res_norm_quant(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* res,
+                        const uint16_t* w, float eps, uint16_t* h, int8_t* xq, float* xs, int Mp, int K,
+                        void* stream);
+
+/* acc INT32 [Mp, 2F] (gate | up) -> per-token INT8 [Mp, F] of swiglu(T(gate), T(up)).
+ * Replaces swiglu_quant, e2e/sc_kernels.py:279-315,585-594. */
+int scmx_swiglu_quant(const int32_t* acc, const float* xscale, const float* wscale, int8_t* xq, float* xs, int Mp,
+                      int F, void* stream);
+
+/* Qwen3 q/k/v split with per-head RMSNorm of q and k, head-major outputs [heads, L, d].  Input is either the INT32
+ * accumulators with their scales (acc != NULL; qkv_epilogue_headnorm, e2e/sc_kernels.py:333-356,597-606) or the T
+ * GEMM output y (qkv_headnorm_y, :359-380,609-616). */
+int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
+                      const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k, uint16_t* v,
+                      int L, int hq, int hk, int d, void* stream);
+
+/* OLMoE q/k/v split with RMSNorm over the full h*d width.  Replaces qkv_fullnorm_y, e2e/sc_kernels.py:390-423,
+ * 629-637. */
+int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q,
+                      uint16_t* k, uint16_t* v, int L, int h, int d, void* stream);
+
+/* ---- decode --------------------------------------------------------------------------------------------------- */
+
+/* W4A8 GEMV on packed weights, `batch` input rows sharing one weight stream (batch 1..8; the reference has batch 1).
+ *   pro 0: xq int8 [batch, K] + xscale [batch];  pro 1: x T[batch, K] quantized in the kernel;
+ *   pro 2: RMSNorm(x, nw, eps) then INT8 in the kernel.
+ *   eidx != NULL (MoE): `slots` output rows, slot j uses expert eidx[j] (or `shared_expert` for the slot after the
+ *   n_eidx routed ones when shared_expert >= 0) and input row j * xstride; batch must be 1.
+ * out: T[slots or batch, N] (epi 1, 2), T[.., N/2] (epi 3).  Replaces gemv, e2e/sc_decode.py:19-183,208-238. */
+int scmx_gemv(const scmx_format* fmt, const void* x, const float* xscale, const uint32_t* codes,
+              const uint8_t* bcodes, const float* wscale, const uint16_t* res, uint16_t* out, int epi, int pro,
+              const uint16_t* nw, float eps, int batch, int N, int K, const int32_t* eidx, int n_eidx, int xstride,
+              int shared_expert, void* stream);
+
+/* ---- mixture of experts ----------------------------------------------------------------------------------------- */
+
+/* Counting sort of the M*topk token-expert assignments by expert: pos [R], tok [R+tm], esorted [R], off [E+1],
+ * tstart [E+1] (tile starts for row tiles of tm).  Replaces route_sort, e2e/sc_moe.py:114-155. */
+int scmx_route_sort(const int32_t* inds, int M, int topk, int n_experts, int tm, int32_t* pos, int32_t* tok,
+                    int32_t* esorted, int32_t* off, int32_t* tstart, void* stream);
+
+/* Grouped W4A8 GEMM over expert segments: rows [off[e], off[e+1]) of the sorted activations use expert e's packed
+ * weights (codes [E, N*K/8], bcodes [E, N, ..], wscale [E, N]).  When `gather` != NULL, sorted row r reads
+ * xq[gather[r]] and xscale[gather[r]] (the xq[tok] gather of e2e/fused_olmoe.py:230 folded into the A-tile load);
+ * otherwise xq / xscale are already in sorted order.  out: INT32 [R,N] (epi 0), T[R,N] (1), T[R,N/2] (3).
+ * Replaces moe_mm, e2e/sc_moe.py:19-92,169-185. */
+int scmx_moe_mm(const scmx_format* fmt, const int8_t* xq, const float* xscale, const int32_t* gather, int R,
+                const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const int32_t* off,
+                const int32_t* tstart, int n_experts, int tm, int N, int K, int epi, void* out, void* stream);
+
+/* The two-pass variant on pre-unpacked INT8 weights [E*N, K].  Replaces moe_mm_i8, e2e/sc_moe.py:95-107,188-200. */
+int scmx_moe_mm_i8(const int8_t* xq, const float* xscale, const int32_t* gather, int R, const int8_t* wq,
+                   const float* wscale, const int32_t* off, const int32_t* tstart, int n_experts, int tm, int N,
+                   int K, int epi, void* out, void* stream);
+
+/* h[t] = res[t] + sum_j T(T(y[pos[t,j]] * score[t,j]) + acc) accumulated sequentially in T; rows >= M copy res.
+ * sscore != NULL: the last slot's score comes from sscore[t] and scores is [M, topk-1] (moe_combine_split).
+ * When xq != NULL also RMSNorm(h, w, eps) + INT8.  Replaces moe_combine / moe_combine_split,
+ * e2e/fused_olmoe.py:34-97. */
+int scmx_moe_combine(const uint16_t* y, const int32_t* pos, const uint16_t* scores, const uint16_t* sscore,
+                     const uint16_t* res, const uint16_t* w, float eps, uint16_t* h, int8_t* xq, float* xs, int M,
+                     int Mp, int K, int topk, void* stream);
+
+/* ---- standard MXFP4 interchange --------------------------------------------------------------------------------- */
+
+/* Standard MXFP4 rows (E2M1 nibbles + one E8M0 byte per 32-block, e8m0 [N, K/32]) -> block codes and row scales of
+ * the default format: shift = e8m0 - min over the row, wscale = 2^(min - 128).  The nibble bytes are used as the
+ * code words unchanged.  status[0] is set to 1 when some row's exponents span more than 3 (not INT8-embeddable).
+ * Device form of the map in e2e/fused_qwen38.py:319-334 (inverse direction) and e2e/gptq_pack.py:29-47. */
+int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SCMX_H */

@@ -1,0 +1,11 @@
+"""scmx: MI355X-native SC-MXFP4 W4A8 linear-layer engine (dense prefill, grouped MoE GEMM, decode GEMV).
+
+Modules keep the names of the reference's kernel call surface so model code can switch imports:
+    sc_format   weight storage descriptor and bit packing
+    sc_kernels  dense prefill kernels (unpack_i8, act_quant, mm_epi, rmsnorm_quant, ...)
+    sc_moe      route_sort, moe_mm, moe_combine
+    sc_decode   gemv
+All compute runs in libscmx.so (hand-written HIP for gfx950); importing the kernels without it raises."""
+from . import _lib, sc_format, sc_kernels, sc_moe, sc_decode  # noqa: F401
+
+__all__ = ["sc_format", "sc_kernels", "sc_moe", "sc_decode"]

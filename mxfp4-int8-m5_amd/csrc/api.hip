@@ -1,0 +1,261 @@
+// Library plumbing (errors, format validation) and the small memory-bound kernels: weight unpack, activation
+// quantization, standard-MXFP4 scale conversion.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "scmx_common.h"
+
+namespace scmx {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: %s", what, hipGetErrorString(e));
+        return SCMX_ERR_LAUNCH;
+    }
+    return SCMX_OK;
+}
+
+int make_dev_format(const scmx_format* f, DevFormat* out) {
+    if (!f) {
+        set_error("format is NULL");
+        return SCMX_ERR_ARG;
+    }
+    const int b = f->block;
+    if (!(b == 8 || b == 16 || b == 32 || b == 64 || b == 128)) {
+        set_error("format: block %d not in {8,16,32,64,128}", b);
+        return SCMX_ERR_FORMAT;
+    }
+    if (!(f->bc_bits == 1 || f->bc_bits == 2 || f->bc_bits == 4 || f->bc_bits == 8) || f->n_mult < 1 ||
+        f->n_mult > 16 || f->n_mult > (1 << f->bc_bits)) {
+        set_error("format: bc_bits %d / n_mult %d unsupported (need bc_bits in {1,2,4,8}, n_mult <= min(16, 2^bc_bits))",
+                  f->bc_bits, f->n_mult);
+        return SCMX_ERR_FORMAT;
+    }
+    int mag_max = 0, mult_max = 0;
+    for (int i = 0; i < 8; ++i) {
+        if (f->code_mag[i] < 0 || f->code_mag[i] > 127) {
+            set_error("format: code_mag[%d] = %d outside 0..127", i, f->code_mag[i]);
+            return SCMX_ERR_FORMAT;
+        }
+        mag_max = f->code_mag[i] > mag_max ? f->code_mag[i] : mag_max;
+    }
+    for (int i = 0; i < f->n_mult; ++i) {
+        if (f->mult[i] < 1 || f->mult[i] > 127) {
+            set_error("format: mult[%d] = %d outside 1..127", i, f->mult[i]);
+            return SCMX_ERR_FORMAT;
+        }
+        mult_max = f->mult[i] > mult_max ? f->mult[i] : mult_max;
+    }
+    if (mag_max * mult_max > 127) {
+        set_error("format: max(code_mag) * max(mult) = %d does not fit INT8", mag_max * mult_max);
+        return SCMX_ERR_FORMAT;
+    }
+    DevFormat d;
+    memset(&d, 0, sizeof(d));
+    for (int i = 0; i < 4; ++i) {
+        d.lut_lo |= uint32_t(f->code_mag[i]) << (8 * i);
+        d.lut_hi |= uint32_t(f->code_mag[4 + i]) << (8 * i);
+    }
+    d.pow2 = 1;
+    for (int i = 0; i < f->n_mult; ++i) {
+        d.mult[i >> 2] |= uint32_t(f->mult[i]) << (8 * (i & 3));
+        if (f->mult[i] != (1 << i)) d.pow2 = 0;
+    }
+    d.block = b;
+    d.block_log2 = b == 8 ? 3 : b == 16 ? 4 : b == 32 ? 5 : b == 64 ? 6 : 7;
+    d.bc_bits = f->bc_bits;
+    *out = d;
+    return SCMX_OK;
+}
+
+// ---- unpack_i8: one thread per 16-byte group of codes (32 weights) ---------------------------------------------
+__global__ __launch_bounds__(256) void unpack_i8_kernel(DevFormat f, const u32x4* __restrict__ codes,
+                                                        const uint8_t* __restrict__ bcodes, u32x4* __restrict__ wq,
+                                                        int64_t n_groups, int groups_per_row, int bc_row_bytes) {
+    const int64_t g = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (g >= n_groups) return;
+    const int64_t row = g / groups_per_row;
+    const uint32_t k0 = uint32_t(g % groups_per_row) * 32u;
+    const u32x4 w = codes[g];
+    const uint8_t* row_bc = bcodes + row * bc_row_bytes;
+    uint32_t o[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t bc = block_code(row_bc, (k0 + 8u * j) >> f.block_log2, f.bc_bits);
+        const BlockLut t = scaled_lut_mul(f.lut_lo, f.lut_hi, mult_of(f, bc));
+        decode_word(w[j], t, o[2 * j], o[2 * j + 1]);
+    }
+    wq[2 * g] = u32x4{o[0], o[1], o[2], o[3]};
+    wq[2 * g + 1] = u32x4{o[4], o[5], o[6], o[7]};
+}
+
+// Fallback for K not a multiple of 32: one thread per code word (8 weights).
+__global__ __launch_bounds__(256) void unpack_i8_word_kernel(DevFormat f, const uint32_t* __restrict__ codes,
+                                                             const uint8_t* __restrict__ bcodes,
+                                                             u32x2* __restrict__ wq, int64_t n_words,
+                                                             int words_per_row, int bc_row_bytes) {
+    const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n_words) return;
+    const int64_t row = i / words_per_row;
+    const uint32_t k0 = uint32_t(i % words_per_row) * 8u;
+    const uint32_t bc = block_code(bcodes + row * bc_row_bytes, k0 >> f.block_log2, f.bc_bits);
+    const BlockLut t = scaled_lut_mul(f.lut_lo, f.lut_hi, mult_of(f, bc));
+    uint32_t a, b;
+    decode_word(codes[i], t, a, b);
+    wq[i] = u32x2{a, b};
+}
+
+// ---- act_quant: one workgroup per token row ---------------------------------------------------------------------
+// Lanes read 8 bf16 (16 bytes) per step; the row maximum goes through LDS; the second sweep re-reads the row
+// (cache hit) and writes 8 codes per lane.
+__global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
+                                                        float* __restrict__ xs, int M, int K) {
+    __shared__ float red[4];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    u32x2* qrow = reinterpret_cast<u32x2*>(xq + size_t(row) * K);
+    if (row >= M) {
+        for (int c = tid; c < K / 8; c += 256) qrow[c] = u32x2{0u, 0u};
+        if (tid == 0) xs[row] = 0.0f;
+        return;
+    }
+    const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
+    float amax = 0.0f;
+    for (int c = tid; c < K / 8; c += 256) {
+        const u32x4 v = xrow[c];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            amax = fmaxf(amax, fabsf(__uint_as_float(v[j] << 16)));
+            amax = fmaxf(amax, fabsf(__uint_as_float(v[j] & 0xFFFF0000u)));
+        }
+    }
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+    for (int c = tid; c < K / 8; c += 256) {
+        const u32x4 v = xrow[c];
+        uint32_t o[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int q0 = quant_code(__uint_as_float(v[j] << 16), qi);
+            const int q1 = quant_code(__uint_as_float(v[j] & 0xFFFF0000u), qi);
+            o[j >> 1] |= (uint32_t(q0) & 0xFFu) << (16 * (j & 1));
+            o[j >> 1] |= (uint32_t(q1) & 0xFFu) << (16 * (j & 1) + 8);
+        }
+        qrow[c] = u32x2{o[0], o[1]};
+    }
+    if (tid == 0) xs[row] = s;
+}
+
+// ---- standard MXFP4 -> block codes + row scale: one wave per row -----------------------------------------------
+__global__ __launch_bounds__(256) void mxfp4_to_sc_kernel(const uint8_t* __restrict__ e8m0,
+                                                          uint8_t* __restrict__ bcodes, float* __restrict__ wscale,
+                                                          int32_t* __restrict__ status, int64_t N, int nb) {
+    const int64_t row = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= N) return;
+    const uint8_t* e = e8m0 + row * nb;
+    int lo = 255, hi = 0;
+    for (int b = lane; b < nb; b += 64) {
+        lo = min(lo, int(e[b]));
+        hi = max(hi, int(e[b]));
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        lo = min(lo, __shfl_xor(lo, off, WAVE));
+        hi = max(hi, __shfl_xor(hi, off, WAVE));
+    }
+    if (hi - lo > 3 && lane == 0) status[0] = 1;
+    for (int byte = lane; byte < nb / 4; byte += 64) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v |= (uint32_t(min(int(e[4 * byte + j]) - lo, 3))) << (2 * j);
+        bcodes[row * (nb / 4) + byte] = uint8_t(v);
+    }
+    // wscale = 2^(lo - 127 - 1); exponents below the normal range give the exact subnormal (or zero) value
+    if (lane == 0) wscale[row] = ldexpf(1.0f, lo - 128);
+}
+
+}  // namespace scmx
+
+using namespace scmx;
+
+extern "C" {
+
+const char* scmx_version(void) { return "scmx 0.1 (gfx950)"; }
+const char* scmx_last_error(void) { return g_err; }
+
+void scmx_default_format(scmx_format* f) {
+    memset(f, 0, sizeof(*f));
+    f->block = 32;
+    f->bc_bits = 2;
+    f->n_mult = 4;
+    const int mag[8] = {0, 1, 2, 3, 4, 6, 8, 12};
+    for (int i = 0; i < 8; ++i) f->code_mag[i] = mag[i];
+    for (int i = 0; i < 4; ++i) f->mult[i] = 1 << i;
+}
+
+int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t* bcodes, int8_t* wq, int64_t n_rows,
+                   int64_t K, void* stream) {
+    DevFormat f;
+    if (int rc = make_dev_format(fmt, &f)) return rc;
+    if (!codes || !bcodes || !wq || n_rows < 0 || K <= 0 || K % f.block || (K / f.block * f.bc_bits) % 8) {
+        set_error("unpack_i8: need non-null pointers, K (%lld) a multiple of block %d and whole block-code bytes per row",
+                  (long long)K, f.block);
+        return SCMX_ERR_ARG;
+    }
+    if (n_rows == 0) return SCMX_OK;
+    const int bc_row_bytes = int(K / f.block * f.bc_bits / 8);
+    hipStream_t s = (hipStream_t)stream;
+    if (K % 32 == 0 && (uintptr_t(codes) % 16 == 0) && (uintptr_t(wq) % 16 == 0)) {
+        const int64_t groups = n_rows * (K / 32);
+        unpack_i8_kernel<<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(
+            f, (const u32x4*)codes, bcodes, (u32x4*)wq, groups, int(K / 32), bc_row_bytes);
+    } else {
+        if (uintptr_t(wq) % 8) {
+            set_error("unpack_i8: output must be 8-byte aligned");
+            return SCMX_ERR_ARG;
+        }
+        const int64_t words = n_rows * (K / 8);
+        unpack_i8_word_kernel<<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s>>>(
+            f, codes, bcodes, (u32x2*)wq, words, int(K / 8), bc_row_bytes);
+    }
+    return check_launch("unpack_i8");
+}
+
+int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream) {
+    if (!x || !xq || !xs || M < 0 || Mp < M || K <= 0 || K % 8 || uintptr_t(x) % 16 || uintptr_t(xq) % 8) {
+        set_error("act_quant: need M <= Mp, K %% 8 == 0 (K = %d), x 16-byte and xq 8-byte aligned", K);
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    act_quant_kernel<<<dim3(Mp), dim3(256), 0, (hipStream_t)stream>>>(x, xq, xs, M, K);
+    return check_launch("act_quant");
+}
+
+int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,
+                     void* stream) {
+    if (!e8m0 || !bcodes || !wscale || !status || N < 0 || K <= 0 || K % 128) {
+        set_error("mxfp4_to_sc: need non-null pointers and K %% 128 == 0 (K = %lld)", (long long)K);
+        return SCMX_ERR_ARG;
+    }
+    if (N == 0) return SCMX_OK;
+    mxfp4_to_sc_kernel<<<dim3((unsigned)((N + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(e8m0, bcodes, wscale,
+                                                                                               status, N, int(K / 32));
+    return check_launch("mxfp4_to_sc");
+}
+
+}  // extern "C"

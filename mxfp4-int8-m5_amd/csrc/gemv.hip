@@ -1,0 +1,292 @@
+// Decode GEMV on packed SC-MXFP4 weights: y[b, n] = epi(xs[b] * ws[n] * sum_k xq[b, k] * q[n, k]).
+//
+// Bandwidth-bound, so no MFMA: a wave owns R consecutive weight rows and walks K in steps of 64 blocks; each lane
+// loads 16 bytes of codes (one run of 32 weights) per row per step, so a wave reads 1 KiB of contiguous weights
+// per load instruction.  Codes are decoded to INT8 four at a time with byte-permute lookups and accumulated with
+// v_dot4_i32_i8 against the INT8 activations, which sit in LDS (one copy per workgroup, bytes of every 8-group
+// stored as elements 0,2,4,6,1,3,5,7 so the decode needs no re-interleave).  All sums are INT32, hence equal to the
+// GEMM's accumulators; the epilogues are the GEMM's.  `BATCH` activation rows share one pass over the weights.
+#include "scmx_common.h"
+
+namespace scmx {
+
+struct GemvArgs {
+    const void* x;            // pro 0: int8 [rows, K]; pro 1, 2: bf16 [rows, K]
+    const float* xscale;      // pro 0
+    const uint32_t* codes;
+    const uint8_t* bcodes;
+    const float* wscale;
+    const uint16_t* res;
+    uint16_t* out;
+    const uint16_t* nw;       // pro 2: RMSNorm weight
+    float eps;
+    int epi, pro, N, K, bc_row_bytes;
+    const int32_t* eidx;      // MoE: expert of each slot
+    int n_eidx, xstride, shared_expert;
+    DevFormat fmt;
+};
+
+__device__ __forceinline__ void store_perm8(int8_t* dst, const int q[8]) {
+    const uint32_t e = (uint32_t(q[0]) & 0xFFu) | ((uint32_t(q[2]) & 0xFFu) << 8) | ((uint32_t(q[4]) & 0xFFu) << 16) |
+                       ((uint32_t(q[6]) & 0xFFu) << 24);
+    const uint32_t o = (uint32_t(q[1]) & 0xFFu) | ((uint32_t(q[3]) & 0xFFu) << 8) | ((uint32_t(q[5]) & 0xFFu) << 16) |
+                       ((uint32_t(q[7]) & 0xFFu) << 24);
+    *reinterpret_cast<u32x2*>(dst) = u32x2{e, o};
+}
+
+// Stage one activation row into LDS as permuted INT8 and return its scale.  `red` holds 66 floats.
+template <int NT>
+__device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.K;
+    if (a.pro == 0) {
+        const u32x2* src = reinterpret_cast<const u32x2*>(reinterpret_cast<const int8_t*>(a.x) + size_t(row) * K);
+        for (int c = tid; c < K / 8; c += NT) {
+            const u32x2 v = src[c];
+            *reinterpret_cast<u32x2*>(sx + 8 * c) = u32x2{perm(v[1], v[0], 0x06040200u), perm(v[1], v[0], 0x07050301u)};
+        }
+        return a.xscale[row];
+    }
+    const uint16_t* xr = reinterpret_cast<const uint16_t*>(a.x) + size_t(row) * K;
+    float inv = 1.0f;
+    if (a.pro == 2) {
+        // sum of squares: K/4 virtual threads of 4 values, 64 virtual threads per wave_sum, then one wave_sum over
+        // the per-group partials (at most 64 groups: K <= 16384)
+        for (int g = wave; g < (K / 4 + 63) / 64; g += NT / 64) {
+            const int v = 64 * g + lane;
+            float ss = 0.0f;
+            if (v < K / 4) {
+                const u32x2 p = *reinterpret_cast<const u32x2*>(xr + 4 * v);
+                const float x0 = __uint_as_float(p[0] << 16), x1 = __uint_as_float(p[0] & 0xFFFF0000u);
+                const float x2 = __uint_as_float(p[1] << 16), x3 = __uint_as_float(p[1] & 0xFFFF0000u);
+                ss = __fadd_rn(ss, __fmul_rn(x0, x0));
+                ss = __fadd_rn(ss, __fmul_rn(x1, x1));
+                ss = __fadd_rn(ss, __fmul_rn(x2, x2));
+                ss = __fadd_rn(ss, __fmul_rn(x3, x3));
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) red[g] = ss;
+        }
+        __syncthreads();
+        if (wave == 0) {
+            const float tot = wave_sum(lane < (K / 4 + 63) / 64 ? red[lane] : 0.0f);
+            if (lane == 0) red[64] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, float(K)), a.eps)));
+        }
+        __syncthreads();
+        inv = red[64];
+        __syncthreads();
+    }
+    auto value = [&](int k) -> float {
+        const float xv = bf16_to_f32(xr[k]);
+        if (a.pro == 2) return round_bf16(__fmul_rn(bf16_to_f32(a.nw[k]), round_bf16(__fmul_rn(xv, inv))));
+        return xv;
+    };
+    float amax = 0.0f;
+    for (int c = tid; c < K / 8; c += NT)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(value(8 * c + i)));
+    amax = wave_max(amax);
+    if (lane == 0) red[wave] = amax;
+    __syncthreads();
+    amax = 0.0f;
+    for (int w = 0; w < NT / 64; ++w) amax = fmaxf(amax, red[w]);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+    for (int c = tid; c < K / 8; c += NT) {
+        int q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(value(8 * c + i), qi);
+        store_perm8(sx + 8 * c, q);
+    }
+    __syncthreads();   // `red` is reused by the next row
+    return s;
+}
+
+template <int BATCH, int R, bool DEFAULT_FMT>
+__global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
+    constexpr int NT = 256;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    int8_t* sx = smem;                                              // [BATCH][K]
+    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * a.K);   // 68 floats
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.K, N = a.N;
+
+    // MoE: one slot per blockIdx.y, its own expert and (xstride = 1) its own input row
+    const int slot = blockIdx.y;
+    int expert = 0, xrow0 = 0;
+    if (a.eidx) {
+        expert = (a.shared_expert >= 0 && slot == a.n_eidx) ? a.shared_expert : a.eidx[slot];
+        xrow0 = slot * a.xstride;
+    }
+    float xs[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) xs[b] = stage_row<NT>(a, xrow0 + b, sx + size_t(b) * K, red);
+    __syncthreads();
+
+    const int n0 = (blockIdx.x * (NT / 64) + wave) * R;
+    if (n0 >= N) return;
+    const size_t erow = size_t(expert) * N;
+    const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + (erow + n0) * (K / 2);
+    const uint8_t* brow = a.bcodes + (erow + n0) * a.bc_row_bytes;
+
+    int acc[R][BATCH];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) acc[r][b] = 0;
+
+    const int nchunk = K / 32;   // 16-byte code groups per row
+    for (int c = lane; c < nchunk; c += 64) {
+        u32x4 w[R];
+        uint32_t bc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            w[r] = *reinterpret_cast<const u32x4*>(crow + size_t(r) * (K / 2) + 16 * c);
+            if (DEFAULT_FMT) bc[r] = (uint32_t(brow[r * a.bc_row_bytes + (c >> 2)]) >> (2 * (c & 3))) & 3u;
+        }
+        u32x4 xv[BATCH][2];
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+            xv[b][0] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32 * c);
+            xv[b][1] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32 * c + 16);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int part[BATCH];
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) part[b] = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint32_t e, o;
+                if (DEFAULT_FMT) {
+                    const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, 0u);   // folds to constants
+                    decode_word_split(w[r][j], t, e, o);
+                } else {
+                    const uint32_t blk = uint32_t(32 * c + 8 * j) >> a.fmt.block_log2;
+                    const uint32_t code = block_code(brow + r * a.bc_row_bytes, blk, a.fmt.bc_bits);
+                    const BlockLut t = scaled_lut_mul(a.fmt.lut_lo, a.fmt.lut_hi, mult_of(a.fmt, code));
+                    decode_word_split(w[r][j], t, e, o);
+                }
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b) {
+                    part[b] = __builtin_amdgcn_sdot4(int(e), int(xv[b][j >> 1][2 * (j & 1)]), part[b], false);
+                    part[b] = __builtin_amdgcn_sdot4(int(o), int(xv[b][j >> 1][2 * (j & 1) + 1]), part[b], false);
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) acc[r][b] += DEFAULT_FMT ? (part[b] << bc[r]) : part[b];
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) acc[r][b] = wave_sum_i32(acc[r][b]);
+    if (lane != 0) return;
+
+    const float* ws = a.wscale + erow + n0;
+    const int orow0 = a.eidx ? slot : 0;
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+        float y[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) y[r] = __fmul_rn(__fmul_rn(float(acc[r][b]), xs[b]), ws[r]);
+        if (a.epi == SCMX_EPI_SCALE) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) a.out[size_t(orow0 + b) * N + n0 + r] = f32_to_bf16(y[r]);
+        } else if (a.epi == SCMX_EPI_RES) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float rv = bf16_to_f32(a.res[size_t(orow0 + b) * N + n0 + r]);
+                a.out[size_t(orow0 + b) * N + n0 + r] = f32_to_bf16(__fadd_rn(rv, round_bf16(y[r])));
+            }
+        } else if (R % 4 == 0) {   // SwiGLU of (g, g, u, u)
+#pragma unroll
+            for (int r = 0; r < R; r += 4) {
+                uint16_t* o = a.out + size_t(orow0 + b) * (N / 2) + (n0 + r) / 2;
+                o[0] = swiglu_bf16(round_bf16(y[r]), round_bf16(y[(r + 2) % R]));
+                o[1] = swiglu_bf16(round_bf16(y[(r + 1) % R]), round_bf16(y[(r + 3) % R]));
+            }
+        }
+    }
+}
+
+template <int BATCH, int R>
+static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
+    const dim3 grid((a.N / R + 3) / 4, slots), block(256);
+    const size_t smem = size_t(BATCH) * a.K + 68 * sizeof(float);
+    if (dflt)
+        gemv_kernel<BATCH, R, true><<<grid, block, smem, s>>>(a);
+    else
+        gemv_kernel<BATCH, R, false><<<grid, block, smem, s>>>(a);
+}
+
+template <int BATCH>
+static void launch_gemv_rows(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
+    // more rows per wave = more loads in flight per lane; fewer = more workgroups for narrow layers
+    const long rows = long(a.N) * slots;
+    if (a.epi == SCMX_EPI_SWIGLU || (rows >= 32768 && a.N % 4 == 0)) return launch_gemv<BATCH, 4>(a, slots, dflt, s);
+    if (rows >= 8192 && a.N % 2 == 0) return launch_gemv<BATCH, 2>(a, slots, dflt, s);
+    return launch_gemv<BATCH, 1>(a, slots, dflt, s);
+}
+
+}  // namespace scmx
+
+using namespace scmx;
+
+extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xscale, const uint32_t* codes,
+                         const uint8_t* bcodes, const float* wscale, const uint16_t* res, uint16_t* out, int epi,
+                         int pro, const uint16_t* nw, float eps, int batch, int N, int K, const int32_t* eidx,
+                         int n_eidx, int xstride, int shared_expert, void* stream) {
+    DevFormat f;
+    if (int rc = make_dev_format(fmt, &f)) return rc;
+    if (!x || !codes || !bcodes || !wscale || !out || (pro == 0 && !xscale) || (pro == 2 && !nw) ||
+        (epi == SCMX_EPI_RES && !res)) {
+        set_error("gemv: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (epi < 1 || epi > 3 || pro < 0 || pro > 2) {
+        set_error("gemv: epilogue %d / prologue %d unknown", epi, pro);
+        return SCMX_ERR_ARG;
+    }
+    if (N <= 0 || K <= 0 || K % 128 || K % f.block || (K / f.block * f.bc_bits) % 8 || (epi == SCMX_EPI_SWIGLU && N % 4)) {
+        set_error("gemv: need K %% 128 == 0, whole block-code bytes per row, N %% 4 == 0 for SwiGLU (N=%d K=%d)", N, K);
+        return SCMX_ERR_ARG;
+    }
+    if (uintptr_t(codes) % 16 || uintptr_t(x) % 8) {
+        set_error("gemv: codes must be 16-byte aligned, x 8-byte aligned");
+        return SCMX_ERR_ARG;
+    }
+    int slots = 1;
+    if (eidx) {
+        if (batch != 1 || n_eidx < 0 || (xstride != 0 && xstride != 1)) {
+            set_error("gemv: the expert-gather form takes batch 1, xstride 0 or 1");
+            return SCMX_ERR_ARG;
+        }
+        slots = n_eidx + (shared_expert >= 0 ? 1 : 0);
+        if (slots == 0) return SCMX_OK;
+    }
+    if (!(batch == 1 || batch == 2 || batch == 4 || batch == 8)) {
+        set_error("gemv: batch %d not in {1,2,4,8}", batch);
+        return SCMX_ERR_ARG;
+    }
+    if (size_t(batch) * K + 68 * sizeof(float) > 64 * 1024) {
+        set_error("gemv: batch * K = %zu bytes of activations exceed the 64 KiB staged per workgroup", size_t(batch) * K);
+        return SCMX_ERR_ARG;
+    }
+    GemvArgs a = {};
+    a.x = x; a.xscale = xscale; a.codes = codes; a.bcodes = bcodes; a.wscale = wscale; a.res = res; a.out = out;
+    a.nw = nw; a.eps = eps; a.epi = epi; a.pro = pro; a.N = N; a.K = K;
+    a.bc_row_bytes = K / f.block * f.bc_bits / 8;
+    a.eidx = eidx; a.n_eidx = n_eidx; a.xstride = xstride; a.shared_expert = eidx ? shared_expert : -1;
+    a.fmt = f;
+    const bool dflt = is_default_format(f);
+    hipStream_t s = (hipStream_t)stream;
+    switch (batch) {
+        case 1: launch_gemv_rows<1>(a, slots, dflt, s); break;
+        case 2: launch_gemv_rows<2>(a, slots, dflt, s); break;
+        case 4: launch_gemv_rows<4>(a, slots, dflt, s); break;
+        default: launch_gemv_rows<8>(a, slots, dflt, s); break;
+    }
+    return check_launch("gemv");
+}

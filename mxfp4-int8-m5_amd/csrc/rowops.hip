@@ -1,0 +1,433 @@
+// Row kernels around the GEMMs (memory-bound, one workgroup per token row): RMSNorm + INT8 quantization, residual
+// epilogue, SwiGLU + quantization, the q/k/v splits with head norms, the MoE token sort and the weighted combine.
+//
+// Reduction order (fixed, so results do not depend on the launch shape): a row's sum of squares is formed by K/4
+// virtual threads of 4 consecutive values summed in order, 64 virtual threads per butterfly wave sum, and one more
+// butterfly over the per-group partials.
+#include "scmx_common.h"
+
+namespace scmx {
+
+constexpr int NT = 256;
+
+// 1 / sqrt(mean(x^2) + eps) of a bf16 row; every thread of the workgroup calls it.  red: >= 65 floats of LDS.
+__device__ float block_inv_rms(const uint16_t* xr, int K, float eps, float* red) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int groups = (K / 4 + 63) / 64;
+    for (int g = wave; g < groups; g += NT / 64) {
+        const int v = 64 * g + lane;
+        float ss = 0.0f;
+        if (v < K / 4) {
+            const u32x2 p = *reinterpret_cast<const u32x2*>(xr + 4 * v);
+            const float x0 = __uint_as_float(p[0] << 16), x1 = __uint_as_float(p[0] & 0xFFFF0000u);
+            const float x2 = __uint_as_float(p[1] << 16), x3 = __uint_as_float(p[1] & 0xFFFF0000u);
+            ss = __fadd_rn(ss, __fmul_rn(x0, x0));
+            ss = __fadd_rn(ss, __fmul_rn(x1, x1));
+            ss = __fadd_rn(ss, __fmul_rn(x2, x2));
+            ss = __fadd_rn(ss, __fmul_rn(x3, x3));
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[g] = ss;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const float tot = wave_sum(lane < groups ? red[lane] : 0.0f);
+        if (lane == 0) red[64] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, float(K)), eps)));
+    }
+    __syncthreads();
+    const float inv = red[64];
+    __syncthreads();
+    return inv;
+}
+
+// Per-token INT8 of a row given as bf16 bit patterns in memory (global or LDS): codes to qrow, scale to *xs.
+__device__ void block_quant_row(const uint16_t* v, int K, int8_t* qrow, float* xs, float* red) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float amax = 0.0f;
+    for (int c = tid; c < K / 4; c += NT) {
+        const u32x2 p = *reinterpret_cast<const u32x2*>(v + 4 * c);
+        amax = fmaxf(amax, fabsf(__uint_as_float(p[0] << 16)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(p[0] & 0xFFFF0000u)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(p[1] << 16)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(p[1] & 0xFFFF0000u)));
+    }
+    amax = wave_max(amax);
+    if (lane == 0) red[wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+    for (int c = tid; c < K / 4; c += NT) {
+        const u32x2 p = *reinterpret_cast<const u32x2*>(v + 4 * c);
+        const int q0 = quant_code(__uint_as_float(p[0] << 16), qi), q1 = quant_code(__uint_as_float(p[0] & 0xFFFF0000u), qi);
+        const int q2 = quant_code(__uint_as_float(p[1] << 16), qi), q3 = quant_code(__uint_as_float(p[1] & 0xFFFF0000u), qi);
+        *reinterpret_cast<uint32_t*>(qrow + 4 * c) = (uint32_t(q0) & 0xFFu) | ((uint32_t(q1) & 0xFFu) << 8) |
+                                                     ((uint32_t(q2) & 0xFFu) << 16) | ((uint32_t(q3) & 0xFFu) << 24);
+    }
+    if (tid == 0) *xs = s;
+    __syncthreads();
+}
+
+__device__ void block_zero_row(int8_t* qrow, float* xs, uint16_t* xn, int K) {
+    for (int c = threadIdx.x; c < K / 4; c += NT) {
+        *reinterpret_cast<uint32_t*>(qrow + 4 * c) = 0u;
+        if (xn) *reinterpret_cast<u32x2*>(xn + 4 * c) = u32x2{0u, 0u};
+    }
+    if (threadIdx.x == 0) *xs = 0.0f;
+}
+
+// y = bf16(w * bf16(x * inv)) for a row, written as bf16 bits to `dst` (LDS) and optionally to xn (global).
+__device__ void block_norm_row(const uint16_t* xr, const uint16_t* w, float inv, uint16_t* dst, uint16_t* xn, int K) {
+    for (int c = threadIdx.x; c < K / 4; c += NT) {
+        const u32x2 p = *reinterpret_cast<const u32x2*>(xr + 4 * c);
+        const u32x2 q = *reinterpret_cast<const u32x2*>(w + 4 * c);
+        uint16_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float xv = __uint_as_float(i & 1 ? (p[i >> 1] & 0xFFFF0000u) : (p[i >> 1] << 16));
+            const float wv = __uint_as_float(i & 1 ? (q[i >> 1] & 0xFFFF0000u) : (q[i >> 1] << 16));
+            o[i] = f32_to_bf16(__fmul_rn(wv, round_bf16(__fmul_rn(xv, inv))));
+        }
+        const u32x2 r = u32x2{uint32_t(o[0]) | (uint32_t(o[1]) << 16), uint32_t(o[2]) | (uint32_t(o[3]) << 16)};
+        *reinterpret_cast<u32x2*>(dst + 4 * c) = r;
+        if (xn) *reinterpret_cast<u32x2*>(xn + 4 * c) = r;
+    }
+    __syncthreads();
+}
+
+// ---- rmsnorm_quant(_n) -----------------------------------------------------------------------------------------
+__global__ __launch_bounds__(NT) void rmsnorm_quant_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                           float eps, int8_t* __restrict__ xq, float* __restrict__ xs,
+                                                           uint16_t* __restrict__ xn, int M, int K) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t srow[];   // K bf16 + 72 floats
+    float* red = reinterpret_cast<float*>(srow + K);
+    const int row = blockIdx.x;
+    int8_t* qrow = xq + size_t(row) * K;
+    uint16_t* nrow = xn ? xn + size_t(row) * K : nullptr;
+    if (row >= M) return block_zero_row(qrow, xs + row, nrow, K);
+    const uint16_t* xr = x + size_t(row) * K;
+    const float inv = block_inv_rms(xr, K, eps, red);
+    block_norm_row(xr, w, inv, srow, nrow, K);
+    block_quant_row(srow, K, qrow, xs + row, red);
+}
+
+// ---- res_norm_quant / res_epilogue -----------------------------------------------------------------------------
+__global__ __launch_bounds__(NT) void res_norm_quant_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
+                                                            const float* __restrict__ wscale, const uint16_t* __restrict__ res,
+                                                            const uint16_t* __restrict__ w, float eps, uint16_t* __restrict__ h,
+                                                            int8_t* __restrict__ xq, float* __restrict__ xs, int K) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t srow[];   // 2 K bf16 + 72 floats
+    uint16_t* hrow_s = srow;
+    uint16_t* nrow_s = srow + K;
+    float* red = reinterpret_cast<float*>(srow + 2 * K);
+    const int row = blockIdx.x;
+    const float xsr = xscale[row];
+    for (int c = threadIdx.x; c < K / 4; c += NT) {
+        const v4i a4 = *reinterpret_cast<const v4i*>(acc + size_t(row) * K + 4 * c);
+        const f32x4 w4 = *reinterpret_cast<const f32x4*>(wscale + 4 * c);
+        const u32x2 r2 = *reinterpret_cast<const u32x2*>(res + size_t(row) * K + 4 * c);
+        uint16_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float y = round_bf16(__fmul_rn(__fmul_rn(float(a4[i]), xsr), w4[i]));
+            const float rv = __uint_as_float(i & 1 ? (r2[i >> 1] & 0xFFFF0000u) : (r2[i >> 1] << 16));
+            o[i] = f32_to_bf16(__fadd_rn(rv, y));
+        }
+        const u32x2 r = u32x2{uint32_t(o[0]) | (uint32_t(o[1]) << 16), uint32_t(o[2]) | (uint32_t(o[3]) << 16)};
+        *reinterpret_cast<u32x2*>(hrow_s + 4 * c) = r;
+        *reinterpret_cast<u32x2*>(h + size_t(row) * K + 4 * c) = r;
+    }
+    __syncthreads();
+    if (!xq) return;
+    const float inv = block_inv_rms(hrow_s, K, eps, red);
+    block_norm_row(hrow_s, w, inv, nrow_s, nullptr, K);
+    block_quant_row(nrow_s, K, xq + size_t(row) * K, xs + row, red);
+}
+
+// ---- swiglu_quant ----------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(NT) void swiglu_quant_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
+                                                          const float* __restrict__ wscale, int8_t* __restrict__ xq,
+                                                          float* __restrict__ xs, int F) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t srow[];   // F bf16 + 72 floats
+    float* red = reinterpret_cast<float*>(srow + F);
+    const int row = blockIdx.x;
+    const float xsr = xscale[row];
+    const int32_t* ar = acc + size_t(row) * 2 * F;
+    for (int c = threadIdx.x; c < F / 4; c += NT) {
+        const v4i g4 = *reinterpret_cast<const v4i*>(ar + 4 * c);
+        const v4i u4 = *reinterpret_cast<const v4i*>(ar + F + 4 * c);
+        const f32x4 wg = *reinterpret_cast<const f32x4*>(wscale + 4 * c);
+        const f32x4 wu = *reinterpret_cast<const f32x4*>(wscale + F + 4 * c);
+        uint16_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float g = round_bf16(__fmul_rn(__fmul_rn(float(g4[i]), xsr), wg[i]));
+            const float u = round_bf16(__fmul_rn(__fmul_rn(float(u4[i]), xsr), wu[i]));
+            o[i] = swiglu_bf16(g, u);
+        }
+        *reinterpret_cast<u32x2*>(srow + 4 * c) =
+            u32x2{uint32_t(o[0]) | (uint32_t(o[1]) << 16), uint32_t(o[2]) | (uint32_t(o[3]) << 16)};
+    }
+    __syncthreads();
+    block_quant_row(srow, F, xq + size_t(row) * F, xs + row, red);
+}
+
+// ---- Qwen3 q/k/v split with per-head RMSNorm: one wave per head, d/64 consecutive values per lane ---------------
+__global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
+                                                          const float* __restrict__ wscale, const uint16_t* __restrict__ y,
+                                                          const uint16_t* __restrict__ qn, const uint16_t* __restrict__ kn,
+                                                          float eps, uint16_t* __restrict__ q, uint16_t* __restrict__ k,
+                                                          uint16_t* __restrict__ v, int L, int hq, int hk, int d) {
+    const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int heads = hq + 2 * hk, ntot = heads * d, per = d / 64;
+    for (int g = wave; g < heads; g += NT / 64) {
+        float yv[8];   // per <= 8 (d <= 512)
+        float ss = 0.0f;
+        for (int i = 0; i < per; ++i) {
+            const int c = g * d + per * lane + i;
+            if (acc)
+                yv[i] = round_bf16(__fmul_rn(__fmul_rn(float(acc[size_t(row) * ntot + c]), xscale[row]), wscale[c]));
+            else
+                yv[i] = bf16_to_f32(y[size_t(row) * ntot + c]);
+            ss = __fadd_rn(ss, __fmul_rn(yv[i], yv[i]));
+        }
+        uint16_t* out;
+        int hh;
+        if (g < hq) { out = q; hh = g; } else if (g < hq + hk) { out = k; hh = g - hq; } else { out = v; hh = g - hq - hk; }
+        uint16_t* o = out + (size_t(hh) * L + row) * d + per * lane;
+        if (g < hq + hk) {
+            ss = wave_sum(ss);
+            const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
+            const uint16_t* w = g < hq ? qn : kn;
+            for (int i = 0; i < per; ++i)
+                o[i] = f32_to_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
+        } else {
+            for (int i = 0; i < per; ++i) o[i] = f32_to_bf16(yv[i]);
+        }
+    }
+}
+
+// ---- OLMoE q/k/v split with RMSNorm over the full h*d width ------------------------------------------------------
+__global__ __launch_bounds__(NT) void qkv_fullnorm_kernel(const uint16_t* __restrict__ y, const uint16_t* __restrict__ qn,
+                                                          const uint16_t* __restrict__ kn, float eps, uint16_t* __restrict__ q,
+                                                          uint16_t* __restrict__ k, uint16_t* __restrict__ v, int L, int h,
+                                                          int d) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t srow[];   // W bf16 + 72 floats
+    const int W = h * d, row = blockIdx.x;
+    float* red = reinterpret_cast<float*>(srow + W);
+    for (int part = 0; part < 3; ++part) {
+        const uint16_t* yr = y + size_t(row) * 3 * W + size_t(part) * W;
+        uint16_t* out = part == 0 ? q : (part == 1 ? k : v);
+        const uint16_t* src = yr;
+        if (part < 2) {
+            const float inv = block_inv_rms(yr, W, eps, red);
+            block_norm_row(yr, part == 0 ? qn : kn, inv, srow, nullptr, W);
+            src = srow;
+        }
+        for (int c = threadIdx.x; c < W / 4; c += NT) {
+            const int col = 4 * c, hh = col / d, dd = col % d;
+            *reinterpret_cast<u32x2*>(out + (size_t(hh) * L + row) * d + dd) = *reinterpret_cast<const u32x2*>(src + col);
+        }
+        __syncthreads();
+    }
+}
+
+// ---- MoE: counting sort of the token-expert assignments, one workgroup ------------------------------------------
+__global__ __launch_bounds__(1024) void route_sort_kernel(const int32_t* __restrict__ inds, int R, int topk, int E, int tm,
+                                                          int32_t* __restrict__ pos, int32_t* __restrict__ tok,
+                                                          int32_t* __restrict__ esorted, int32_t* __restrict__ off,
+                                                          int32_t* __restrict__ tstart) {
+    __shared__ uint32_t cnt[1024], cur[1024], tl[1024];
+    const int tid = threadIdx.x;
+    cnt[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < R; i += 1024) atomicAdd(&cnt[min(max(inds[i], 0), E - 1)], 1u);
+    __syncthreads();
+    // exclusive prefix sums of the counts and of the per-expert tile counts (Hillis-Steele over 1024 entries)
+    const uint32_t c = tid < E ? cnt[tid] : 0u;
+    uint32_t so = c, st = (c + tm - 1) / tm;
+    const uint32_t t0 = st;
+    cur[tid] = so;
+    tl[tid] = st;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const uint32_t ao = tid >= d ? cur[tid - d] : 0u, at = tid >= d ? tl[tid - d] : 0u;
+        __syncthreads();
+        so += ao;
+        st += at;
+        cur[tid] = so;
+        tl[tid] = st;
+        __syncthreads();
+    }
+    if (tid < E) {
+        off[tid] = int32_t(so - c);
+        tstart[tid] = int32_t(st - t0);
+    }
+    if (tid == E - 1) {
+        off[E] = int32_t(so);
+        tstart[E] = int32_t(st);
+    }
+    __syncthreads();
+    cur[tid] = so - c;   // next free row of each expert
+    __syncthreads();
+    for (int i = tid; i < R; i += 1024) {
+        const int e = min(max(inds[i], 0), E - 1);
+        const uint32_t p = atomicAdd(&cur[e], 1u);
+        pos[i] = int32_t(p);
+        tok[p] = i / topk;
+        esorted[p] = e;
+    }
+    for (int p = R + tid; p < R + tm; p += 1024) tok[p] = 0;   // padding rows gather token 0
+}
+
+// ---- MoE: weighted combine of the top-k expert outputs, sequential in bf16 ---------------------------------------
+__global__ __launch_bounds__(NT) void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ pos,
+                                                         const uint16_t* __restrict__ scores, const uint16_t* __restrict__ sscore,
+                                                         const uint16_t* __restrict__ res, const uint16_t* __restrict__ w,
+                                                         float eps, uint16_t* __restrict__ h, int8_t* __restrict__ xq,
+                                                         float* __restrict__ xs, int M, int K, int topk) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t srow[];   // 2 K bf16 + 72 floats
+    uint16_t* hrow_s = srow;
+    uint16_t* nrow_s = srow + K;
+    float* red = reinterpret_cast<float*>(srow + 2 * K);
+    const int row = blockIdx.x;
+    const int nsc = sscore ? topk - 1 : topk;
+    for (int c = threadIdx.x; c < K / 4; c += NT) {
+        const u32x2 r2 = *reinterpret_cast<const u32x2*>(res + size_t(row) * K + 4 * c);
+        u32x2 o = r2;
+        if (row < M) {
+            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int j = 0; j < topk; ++j) {
+                const int p = pos[row * topk + j];
+                const float sc = bf16_to_f32((sscore && j == topk - 1) ? sscore[row] : scores[row * nsc + j]);
+                const u32x2 y2 = *reinterpret_cast<const u32x2*>(y + size_t(p) * K + 4 * c);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float yv = __uint_as_float(i & 1 ? (y2[i >> 1] & 0xFFFF0000u) : (y2[i >> 1] << 16));
+                    acc[i] = round_bf16(__fadd_rn(round_bf16(__fmul_rn(yv, sc)), acc[i]));
+                }
+            }
+            uint16_t hb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float rv = __uint_as_float(i & 1 ? (r2[i >> 1] & 0xFFFF0000u) : (r2[i >> 1] << 16));
+                hb[i] = f32_to_bf16(__fadd_rn(rv, acc[i]));
+            }
+            o = u32x2{uint32_t(hb[0]) | (uint32_t(hb[1]) << 16), uint32_t(hb[2]) | (uint32_t(hb[3]) << 16)};
+        }
+        *reinterpret_cast<u32x2*>(hrow_s + 4 * c) = o;
+        *reinterpret_cast<u32x2*>(h + size_t(row) * K + 4 * c) = o;
+    }
+    __syncthreads();
+    if (!xq) return;
+    const float inv = block_inv_rms(hrow_s, K, eps, red);
+    block_norm_row(hrow_s, w, inv, nrow_s, nullptr, K);
+    block_quant_row(nrow_s, K, xq + size_t(row) * K, xs + row, red);
+}
+
+static bool row_shape_ok(const char* who, int rows, int K, int max_k) {
+    if (rows < 0 || K <= 0 || K % 4 || K > max_k) {
+        set_error("%s: need rows >= 0 and K %% 4 == 0, K <= %d (rows=%d K=%d)", who, max_k, rows, K);
+        return false;
+    }
+    return true;
+}
+
+}  // namespace scmx
+
+using namespace scmx;
+
+extern "C" {
+
+int scmx_rmsnorm_quant(const uint16_t* x, const uint16_t* w, float eps, int8_t* xq, float* xs, uint16_t* xn, int M,
+                       int Mp, int K, void* stream) {
+    if (!x || !w || !xq || !xs || Mp < M || !row_shape_ok("rmsnorm_quant", M, K, 16384)) {
+        if (!(x && w && xq && xs) || Mp < M) set_error("rmsnorm_quant: null pointer or Mp < M");
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    rmsnorm_quant_kernel<<<dim3(Mp), dim3(NT), size_t(K) * 2 + 72 * 4, (hipStream_t)stream>>>(x, w, eps, xq, xs, xn, M, K);
+    return check_launch("rmsnorm_quant");
+}
+
+int scmx_res_norm_quant(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* res,
+                        const uint16_t* w, float eps, uint16_t* h, int8_t* xq, float* xs, int Mp, int K, void* stream) {
+    if (!acc || !xscale || !wscale || !res || !h || (xq && (!w || !xs)) || !row_shape_ok("res_norm_quant", Mp, K, 8192)) {
+        if (!(acc && xscale && wscale && res && h) || (xq && (!w || !xs))) set_error("res_norm_quant: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    res_norm_quant_kernel<<<dim3(Mp), dim3(NT), size_t(K) * 4 + 72 * 4, (hipStream_t)stream>>>(acc, xscale, wscale, res, w,
+                                                                                                  eps, h, xq, xs, K);
+    return check_launch("res_norm_quant");
+}
+
+int scmx_swiglu_quant(const int32_t* acc, const float* xscale, const float* wscale, int8_t* xq, float* xs, int Mp, int F,
+                      void* stream) {
+    if (!acc || !xscale || !wscale || !xq || !xs || !row_shape_ok("swiglu_quant", Mp, F, 16384)) {
+        if (!(acc && xscale && wscale && xq && xs)) set_error("swiglu_quant: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    swiglu_quant_kernel<<<dim3(Mp), dim3(NT), size_t(F) * 2 + 72 * 4, (hipStream_t)stream>>>(acc, xscale, wscale, xq, xs, F);
+    return check_launch("swiglu_quant");
+}
+
+int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
+                      const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k, uint16_t* v, int L,
+                      int hq, int hk, int d, void* stream) {
+    if ((!acc && !y) || (acc && (!xscale || !wscale)) || !qn || !kn || !q || !k || !v) {
+        set_error("qkv_headnorm: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (L < 0 || hq < 1 || hk < 1 || d % 64 || d < 64 || d > 512) {
+        set_error("qkv_headnorm: need head dim a multiple of 64 in 64..512 (d=%d)", d);
+        return SCMX_ERR_ARG;
+    }
+    if (L == 0) return SCMX_OK;
+    qkv_headnorm_kernel<<<dim3(L), dim3(NT), 0, (hipStream_t)stream>>>(acc, xscale, wscale, y, qn, kn, eps, q, k, v, L, hq,
+                                                                        hk, d);
+    return check_launch("qkv_headnorm");
+}
+
+int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k,
+                      uint16_t* v, int L, int h, int d, void* stream) {
+    if (!y || !qn || !kn || !q || !k || !v) {
+        set_error("qkv_fullnorm: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (L < 0 || h < 1 || d % 4 || !row_shape_ok("qkv_fullnorm", L, h * d, 16384)) return SCMX_ERR_ARG;
+    if (L == 0) return SCMX_OK;
+    qkv_fullnorm_kernel<<<dim3(L), dim3(NT), size_t(h) * d * 2 + 72 * 4, (hipStream_t)stream>>>(y, qn, kn, eps, q, k, v, L,
+                                                                                                 h, d);
+    return check_launch("qkv_fullnorm");
+}
+
+int scmx_route_sort(const int32_t* inds, int M, int topk, int n_experts, int tm, int32_t* pos, int32_t* tok,
+                    int32_t* esorted, int32_t* off, int32_t* tstart, void* stream) {
+    if (!inds || !pos || !tok || !esorted || !off || !tstart || M < 0 || topk < 1 || tm < 1 || n_experts < 1 ||
+        n_experts > 1024) {
+        set_error("route_sort: null pointer, or n_experts (%d) outside 1..1024", n_experts);
+        return SCMX_ERR_ARG;
+    }
+    route_sort_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>(inds, M * topk, topk, n_experts, tm, pos, tok,
+                                                                        esorted, off, tstart);
+    return check_launch("route_sort");
+}
+
+int scmx_moe_combine(const uint16_t* y, const int32_t* pos, const uint16_t* scores, const uint16_t* sscore,
+                     const uint16_t* res, const uint16_t* w, float eps, uint16_t* h, int8_t* xq, float* xs, int M, int Mp,
+                     int K, int topk, void* stream) {
+    if (!y || !pos || !scores || !res || !h || (xq && (!w || !xs)) || Mp < M || topk < 1 ||
+        !row_shape_ok("moe_combine", M, K, 8192)) {
+        if (!(y && pos && scores && res && h) || (xq && (!w || !xs)) || Mp < M || topk < 1)
+            set_error("moe_combine: null pointer argument, Mp < M or topk < 1");
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    moe_combine_kernel<<<dim3(Mp), dim3(NT), size_t(K) * 4 + 72 * 4, (hipStream_t)stream>>>(y, pos, scores, sscore, res, w,
+                                                                                             eps, h, xq, xs, M, K, topk);
+    return check_launch("moe_combine");
+}
+
+}  // extern "C"

@@ -1,0 +1,43 @@
+"""Decode GEMV call surface (the reference's e2e/sc_decode.py) on torch tensors over libscmx.so.
+
+`gemv` keeps the reference's signature; `rows` / `vpl` / `nsg` / `splitk` are accepted as hints (the kernel picks its
+own launch shape and the result never depends on it).  New here: a 2-D `xq` [B, K] without `eidx` runs B input rows
+against one pass over the weights (batch 2, 4 or 8) and returns [B, N]."""
+import torch
+
+from . import _lib
+from . import sc_format as F
+from . import sc_kernels as S
+
+GEMV_TILE = (4, 16, 2)
+GEMV_TILES = {}
+
+
+def gemv(xq, codes, bcodes, xscale, wscale, N, epi, dtype=torch.bfloat16, res=None, nsg=None, eidx=None, xstride=0,
+         pro=0, nw=None, eps=None, rows=None, vpl=None, shared=None, splitk=None, fmt=None):
+    """W4A8 GEMV.  pro=0: xq int8 [K] (or rows) with xscale; pro=1: xq is a bf16 row quantized in the kernel;
+    pro=2: RMSNorm(nw, eps) + INT8 in the kernel.  Output EPI 1: [N]; 2: [N] = res + y; 3: [N/2].
+    MoE (eidx int32 [S]): codes [E, ..], wscale [E, N]; slot j uses expert eidx[j] and input row j if xstride=1;
+    shared=e adds one slot for expert e -> [S(+1), N or N/2]."""
+    S._check_dtype(dtype)
+    fmt = fmt or F.DEFAULT
+    K = xq.shape[-1]
+    no = N // 2 if epi == 3 else N
+    batch, nslot = 1, 0
+    if eidx is not None:
+        nslot = eidx.numel()
+        slots = nslot + (shared is not None)
+        eidx = eidx if eidx.dtype == torch.int32 else eidx.view(torch.int32) if eidx.element_size() == 4 else eidx.to(torch.int32)
+        out = torch.empty((slots, no), dtype=torch.bfloat16, device=xq.device)
+    elif xq.dim() == 2 and xq.shape[0] > 1:
+        batch = xq.shape[0]
+        out = torch.empty((batch, no), dtype=torch.bfloat16, device=xq.device)
+    else:
+        out = torch.empty(no, dtype=torch.bfloat16, device=xq.device)
+    assert (pro == 0 and xq.dtype == torch.int8) or (pro in (1, 2) and xq.dtype == torch.bfloat16)
+    _lib.call("scmx_gemv", fmt.c_struct(), _lib.ptr(xq), _lib.ptr(xscale) if pro == 0 else None, _lib.ptr(codes),
+              _lib.ptr(bcodes), _lib.ptr(wscale), _lib.ptr(res) if epi == 2 else None, _lib.ptr(out), epi, pro,
+              _lib.ptr(nw) if pro == 2 else None, S._eps(eps) if pro == 2 else 0.0, batch, N, K,
+              _lib.ptr(eidx) if eidx is not None else None, nslot, xstride, -1 if shared is None else int(shared),
+              _lib.stream())
+    return out

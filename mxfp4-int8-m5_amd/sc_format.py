@@ -1,0 +1,98 @@
+"""Storage format of the 4-bit weights, host side: the descriptor the kernels are called with and the bit-packing
+of already-quantized codes.  Mirrors the interface of the reference's e2e/sc_format.py (Format, DEFAULT, pack_rows,
+from_shift_layout); decoding runs on the GPU (sc_kernels.unpack_i8).
+
+Layouts (row-major over N, K contiguous):
+  codes   uint32 [N*K/8]   element k = 8j+i in bits 4i..4i+3 of word j; code = sign<<3 | index into code_mag
+  bcodes  uint8 [N, K*bc_bits/(8*block)]   block b in bits bc_bits*(b % per_byte) of byte b // per_byte
+  wscale  f32 [N]
+"""
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+@dataclass(frozen=True)
+class Format:
+    block: int = 32
+    code_mag: tuple = (0, 1, 2, 3, 4, 6, 8, 12)
+    mult: tuple = (1, 2, 4, 8)
+    bc_bits: int = 2
+    inline_mult: bool = False   # accepted for interface compatibility; the kernels need no such hint
+
+    def __post_init__(self):
+        assert self.block % 8 == 0, "one code word (8 weights) must lie in one block"
+        assert self.bc_bits in (1, 2, 4, 8) and len(self.mult) <= 2 ** self.bc_bits
+        assert len(self.code_mag) == 8 and max(self.code_mag) * max(self.mult) <= 127, "must fit INT8"
+
+    @property
+    def per_byte(self):
+        return 8 // self.bc_bits
+
+    def bits_per_weight(self, K):
+        return 4 + self.bc_bits / self.block + 32 / K
+
+    def c_struct(self):
+        """The scmx_format passed across the C ABI."""
+        if len(self.mult) > 16:
+            raise ValueError("the kernels take at most 16 block multipliers")
+        f = _lib.CFormat()
+        f.block, f.bc_bits, f.n_mult = self.block, self.bc_bits, len(self.mult)
+        for i, v in enumerate(self.code_mag):
+            f.code_mag[i] = int(v)
+        for i, v in enumerate(self.mult):
+            f.mult[i] = int(v)
+        return f
+
+
+DEFAULT = Format()
+
+
+def _pack_bcodes(bcode, fmt):
+    n, nb = bcode.shape
+    assert nb % fmt.per_byte == 0
+    grp = bcode.astype(np.uint32).reshape(n, nb // fmt.per_byte, fmt.per_byte)
+    return (grp << (np.arange(fmt.per_byte, dtype=np.uint32) * fmt.bc_bits)).sum(-1).astype(np.uint8)
+
+
+def pack_rows(code4, bcode, wscale, fmt=None):
+    """code4 uint8 [N, K] (sign << 3 | idx), bcode uint8 [N, K/block], wscale [N] -> (codes, bcodes, wscale)."""
+    fmt = fmt or DEFAULT
+    n, k = code4.shape
+    assert k % fmt.block == 0 and bcode.max(initial=0) < len(fmt.mult)
+    c = code4.astype(np.uint32).reshape(n, k // 8, 8)
+    codes = (c << (np.arange(8, dtype=np.uint32) * 4)).sum(-1, dtype=np.uint32).reshape(-1)
+    return codes, _pack_bcodes(np.asarray(bcode, np.uint8), fmt), np.asarray(wscale, np.float32)
+
+
+def from_shift_layout(codes_u32, shifts, wscale, fmt=None):
+    """Byte-shift layout (codes, shifts uint8 [N, K/32] in 0..3, wscale) -> packed block codes; no requantization."""
+    fmt = fmt or DEFAULT
+    assert tuple(fmt.mult) == (1, 2, 4, 8), "the shift layout is the power-of-two format"
+    return (np.asarray(codes_u32, np.uint32).reshape(-1), _pack_bcodes(np.asarray(shifts, np.uint8), fmt),
+            np.asarray(wscale, np.float32))
+
+
+def to_device(codes, bcodes, wscale, device="cuda"):
+    """numpy packed arrays -> torch tensors (codes as int32 bit patterns; torch has no uint32 arithmetic)."""
+    return (torch.from_numpy(np.ascontiguousarray(codes, np.uint32).view(np.int32)).to(device),
+            torch.from_numpy(np.ascontiguousarray(bcodes, np.uint8)).to(device),
+            torch.from_numpy(np.ascontiguousarray(wscale, np.float32)).to(device))
+
+
+def from_mxfp4(nibbles, e8m0):
+    """Standard MXFP4 on the GPU: nibbles uint8 [N, K/2] (E2M1 codes, even k low) and E8M0 uint8 [N, K/32] ->
+    (codes, bcodes, wscale) of the default format.  Raises if a row's exponents span more than 3."""
+    n, nb = e8m0.shape
+    k = nb * 32
+    assert nibbles.shape == (n, k // 2) and nibbles.dtype == torch.uint8 and e8m0.dtype == torch.uint8
+    bc = torch.empty((n, nb // 4), dtype=torch.uint8, device=e8m0.device)
+    ws = torch.empty(n, dtype=torch.float32, device=e8m0.device)
+    status = torch.zeros(1, dtype=torch.int32, device=e8m0.device)
+    _lib.call("scmx_mxfp4_to_sc", _lib.ptr(e8m0), _lib.ptr(bc), _lib.ptr(ws), _lib.ptr(status), n, k, _lib.stream())
+    if int(status.item()):
+        raise ValueError("a row's block exponents span more than 3: not INT8-embeddable")
+    return nibbles.contiguous().view(torch.int32).reshape(-1), bc, ws

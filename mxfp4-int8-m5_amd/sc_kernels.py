@@ -1,0 +1,213 @@
+"""Dense prefill call surface: the function names, argument order and defaults of the reference's e2e/sc_kernels.py,
+on torch (ROCm) tensors, backed by the HIP kernels of libscmx.so through its C ABI.
+
+Conventions kept from the reference (e2e/sc_kernels.py:15-17): kernels take M rows and write Mp >= M rows, rows >= M
+are zero; `deps` is accepted and ignored (it only ordered MLX's lazy graph — HIP streams are already ordered);
+`tile` / `nt` are accepted as hints and never change a result.  `eps` may be a float or a 1-element tensor.
+
+Difference by design: `unpack_i8` may return a `PackedWq` handle instead of an INT8 tensor (FUSE_UNPACK, default on).
+`mm_epi` / `mm_i8_i32` given that handle run the GEMM whose workgroups unpack their weight tile in LDS, so the INT8
+weights are never written to memory; `handle.materialize()` (or lazy=False) gives the reference's INT8 tensor.
+"""
+import numpy as np
+import torch
+
+from . import _lib
+from . import sc_format as F
+
+TM, TN, NSG, GROUP_M = 128, 64, 4, 8     # the reference's default tile (kept for pad_rows and as accepted hints)
+FUSE_UNPACK = True
+
+
+def set_format(fmt):
+    """Switch the default weight format of every wrapper (the C ABI itself takes the format per call)."""
+    F.DEFAULT = fmt
+
+
+def pad_rows(M):
+    return -(-M // TM) * TM
+
+
+def _eps(eps):
+    return float(eps) if not torch.is_tensor(eps) else float(eps.reshape(-1)[0].item())
+
+
+def _check_dtype(dtype):
+    if dtype not in (torch.bfloat16, None):
+        raise ValueError("the kernels emit bfloat16 (the reference's model dtype)")
+
+
+class PackedWq:
+    """Packed weights standing in for the INT8 tensor unpack_i8 would produce."""
+
+    def __init__(self, codes, bcodes, N, K, fmt):
+        self.codes, self.bcodes, self.N, self.K, self.fmt = codes, bcodes, N, K, fmt
+        self.shape, self.dtype, self.device = (N, K), torch.int8, codes.device
+
+    def materialize(self):
+        return unpack_i8(self.codes, self.bcodes, self.N, self.K, lazy=False, fmt=self.fmt)
+
+    def __getitem__(self, idx):          # row selection / permutation, as callers do on the INT8 tensor
+        return self.materialize()[idx]
+
+    def cpu(self):
+        return self.materialize().cpu()
+
+
+def unpack_i8(codes, bcodes, N, K, deps=(), lazy=None, fmt=None):
+    """Packed codes (flat, 4-byte ints) + block codes uint8 [N, ..] -> INT8 [N, K]."""
+    fmt = fmt or F.DEFAULT
+    if FUSE_UNPACK if lazy is None else lazy:
+        return PackedWq(codes, bcodes, N, K, fmt)
+    assert codes.numel() * codes.element_size() == N * K // 2, "codes must hold N*K/2 bytes"
+    wq = torch.empty((N, K), dtype=torch.int8, device=codes.device)
+    _lib.call("scmx_unpack_i8", fmt.c_struct(), _lib.ptr(codes), _lib.ptr(bcodes), _lib.ptr(wq), N, K, _lib.stream())
+    return wq
+
+
+def act_quant(x, Mp=None, nt=256, deps=()):
+    """Per-token symmetric INT8: x bf16 [M, K] -> (xq int8 [Mp, K], xscale f32 [Mp]); rows >= M zero."""
+    M, K = x.shape
+    Mp = Mp or pad_rows(M)
+    assert x.dtype == torch.bfloat16
+    xq = torch.empty((Mp, K), dtype=torch.int8, device=x.device)
+    xs = torch.empty(Mp, dtype=torch.float32, device=x.device)
+    _lib.call("scmx_act_quant", _lib.ptr(x), _lib.ptr(xq), _lib.ptr(xs), M, Mp, K, _lib.stream())
+    return xq, xs
+
+
+def _gemm(xq, wq, xscale, wscale, epi, res):
+    (M, K), N = xq.shape, wq.shape[0]
+    assert xq.dtype == torch.int8 and wq.shape[1] == K
+    if epi == 0:
+        out = torch.empty((M, N), dtype=torch.int32, device=xq.device)
+    else:
+        out = torch.empty((M, N // 2 if epi == 3 else N), dtype=torch.bfloat16, device=xq.device)
+    if epi == 2:
+        assert res is not None and tuple(res.shape) == (M, N) and res.dtype == torch.bfloat16
+    r = _lib.ptr(res) if epi == 2 else None
+    if isinstance(wq, PackedWq):
+        _lib.call("scmx_mm_w4a8", wq.fmt.c_struct(), _lib.ptr(xq), _lib.ptr(xscale), _lib.ptr(wq.codes),
+                  _lib.ptr(wq.bcodes), _lib.ptr(wscale), r, _lib.ptr(out), epi, M, N, K, _lib.stream())
+    else:
+        assert wq.dtype == torch.int8
+        _lib.call("scmx_mm_epi", _lib.ptr(xq), _lib.ptr(wq), _lib.ptr(xscale), _lib.ptr(wscale), r, _lib.ptr(out), epi,
+                  M, N, K, _lib.stream())
+    return out
+
+
+def mm_i8_i32(xq, wq, deps=(), tile=None):
+    """INT8 [M, K] x INT8 [N, K]^T -> INT32 [M, N] (wq: INT8 tensor or PackedWq)."""
+    return _gemm(xq, wq, None, None, 0, None)
+
+
+def mm_epi(xq, wq, xscale, wscale, epi, dtype=torch.bfloat16, res=None, deps=(), tile=None):
+    """INT8 GEMM + in-register epilogue (EPI 1: scaled bf16, 2: + residual, 3: swiglu of interleaved gate/up)."""
+    _check_dtype(dtype)
+    assert epi in (1, 2, 3)
+    return _gemm(xq, wq, xscale, wscale, epi, res)
+
+
+def linear_w4a8(x, codes, bcodes, wscale, N, epi=1, res=None, fmt=None, workspace=None):
+    """One call for a whole W4A8 linear on bf16 activations [M, K]: the activation-quantization prologue and the
+    fused-unpack GEMM are enqueued by a single C entry point (scmx_linear_w4a8).  Returns bf16 [M, N or N/2]."""
+    fmt = fmt or F.DEFAULT
+    M, K = x.shape
+    assert x.dtype == torch.bfloat16 and epi in (1, 2, 3)
+    need = _lib.load().scmx_linear_w4a8_workspace(M, K)
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    out = torch.empty((M, N // 2 if epi == 3 else N), dtype=torch.bfloat16, device=x.device)
+    _lib.call("scmx_linear_w4a8", fmt.c_struct(), _lib.ptr(x), _lib.ptr(codes), _lib.ptr(bcodes), _lib.ptr(wscale),
+              _lib.ptr(res) if epi == 2 else None, _lib.ptr(out), epi, M, N, K, _lib.ptr(workspace),
+              workspace.numel() * workspace.element_size(), _lib.stream())
+    return out
+
+
+def interleave_gate_up(F_):
+    """Row permutation of [gate (F rows); up (F rows)] into groups g_2p, g_2p+1, u_2p, u_2p+1 for EPI 3."""
+    p = np.arange(F_ // 2)
+    return np.stack([2 * p, 2 * p + 1, F_ + 2 * p, F_ + 2 * p + 1], 1).reshape(-1)
+
+
+def _rms(x, w, eps, Mp, want_xn):
+    M, K = x.shape
+    Mp = Mp or pad_rows(M)
+    assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    xq = torch.empty((Mp, K), dtype=torch.int8, device=x.device)
+    xs = torch.empty(Mp, dtype=torch.float32, device=x.device)
+    xn = torch.empty((Mp, K), dtype=torch.bfloat16, device=x.device) if want_xn else None
+    _lib.call("scmx_rmsnorm_quant", _lib.ptr(x), _lib.ptr(w), _eps(eps), _lib.ptr(xq), _lib.ptr(xs), _lib.ptr(xn), M, Mp,
+              K, _lib.stream())
+    return (xq, xs, xn) if want_xn else (xq, xs)
+
+
+def rmsnorm_quant(x, w, eps, Mp=None, deps=()):
+    """x [M, K] -> (xq int8 [Mp, K], xscale f32 [Mp]) of rms_norm(x, w, eps)."""
+    return _rms(x, w, eps, Mp, False)
+
+
+def rmsnorm_quant_n(x, w, eps, Mp=None, deps=()):
+    """rmsnorm_quant that also returns the normalized bf16 rows: (xq, xscale, xn [Mp, K])."""
+    return _rms(x, w, eps, Mp, True)
+
+
+def res_norm_quant(acc, xscale, wscale, res, w, eps, deps=()):
+    """h = res + bf16(acc * xscale * wscale); returns (h [Mp, K], xq, xscale') of rms_norm(h)."""
+    Mp, K = acc.shape
+    assert tuple(res.shape) == (Mp, K) and acc.dtype == torch.int32
+    h = torch.empty_like(res)
+    xq = torch.empty((Mp, K), dtype=torch.int8, device=acc.device)
+    xs = torch.empty(Mp, dtype=torch.float32, device=acc.device)
+    _lib.call("scmx_res_norm_quant", _lib.ptr(acc), _lib.ptr(xscale), _lib.ptr(wscale), _lib.ptr(res), _lib.ptr(w),
+              _eps(eps), _lib.ptr(h), _lib.ptr(xq), _lib.ptr(xs), Mp, K, _lib.stream())
+    return h, xq, xs
+
+
+def res_epilogue(acc, xscale, wscale, res, deps=()):
+    """h = res + bf16(acc * xscale * wscale)."""
+    Mp, N = acc.shape
+    h = torch.empty_like(res)
+    _lib.call("scmx_res_norm_quant", _lib.ptr(acc), _lib.ptr(xscale), _lib.ptr(wscale), _lib.ptr(res), None, 0.0,
+              _lib.ptr(h), None, None, Mp, N, _lib.stream())
+    return h
+
+
+def swiglu_quant(acc, xscale, wscale, dtype=torch.bfloat16, nt=512, deps=()):
+    """acc [Mp, 2F] (gate | up) -> (xq int8 [Mp, F], xscale f32 [Mp]) of swiglu(bf16 gate, bf16 up)."""
+    _check_dtype(dtype)
+    Mp, F2 = acc.shape
+    Fh = F2 // 2
+    xq = torch.empty((Mp, Fh), dtype=torch.int8, device=acc.device)
+    xs = torch.empty(Mp, dtype=torch.float32, device=acc.device)
+    _lib.call("scmx_swiglu_quant", _lib.ptr(acc), _lib.ptr(xscale), _lib.ptr(wscale), _lib.ptr(xq), _lib.ptr(xs), Mp, Fh,
+              _lib.stream())
+    return xq, xs
+
+
+def _headnorm(acc, xscale, wscale, y, qn, kn, eps, L, hq, hk, d, dev):
+    q = torch.empty((hq, L, d), dtype=torch.bfloat16, device=dev)
+    k = torch.empty((hk, L, d), dtype=torch.bfloat16, device=dev)
+    v = torch.empty((hk, L, d), dtype=torch.bfloat16, device=dev)
+    _lib.call("scmx_qkv_headnorm", _lib.ptr(acc), _lib.ptr(xscale), _lib.ptr(wscale), _lib.ptr(y), _lib.ptr(qn),
+              _lib.ptr(kn), _eps(eps), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), L, hq, hk, d, _lib.stream())
+    return q, k, v
+
+
+def qkv_epilogue_headnorm(acc, xscale, wscale, qn, kn, eps, L, hq, hk, d, dtype=torch.bfloat16, deps=()):
+    """Qwen3: acc [Mp, (hq + 2 hk) d] -> q [hq, L, d], k [hk, L, d], v [hk, L, d] (q/k per-head RMSNorm)."""
+    _check_dtype(dtype)
+    return _headnorm(acc, xscale, wscale, None, qn, kn, eps, L, hq, hk, d, acc.device)
+
+
+def qkv_headnorm_y(y, qn, kn, eps, L, hq, hk, d, deps=()):
+    """Qwen3: bf16 y [Mp, (hq + 2 hk) d] -> q, k, v head-major with per-head RMSNorm of q and k."""
+    return _headnorm(None, None, None, y, qn, kn, eps, L, hq, hk, d, y.device)
+
+
+def qkv_fullnorm_y(y, qn, kn, eps, L, h, d, deps=()):
+    """OLMoE: bf16 y [Mp, 3 h d] -> q, k, v [h, L, d] with RMSNorm over the full h*d-wide q and k."""
+    q, k, v = (torch.empty((h, L, d), dtype=torch.bfloat16, device=y.device) for _ in range(3))
+    _lib.call("scmx_qkv_fullnorm", _lib.ptr(y), _lib.ptr(qn), _lib.ptr(kn), _eps(eps), _lib.ptr(q), _lib.ptr(k),
+              _lib.ptr(v), L, h, d, _lib.stream())
+    return q, k, v

@@ -1,0 +1,165 @@
+"""Dense prefill parity on the GPU, through the C ABI: unpack, activation quantization, INT32 GEMM (bit-exact) and
+the scaling epilogues, against the numpy oracle.  Mirrors e2e/test_sc_kernels.py:33-51,121-157 and
+e2e/test_formats.py:26-36 of the reference."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bf16, layout, linear
+from tests.util import FORMATS, dev, host, llm_acts, llm_weights, product_format, random_packed
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def S():
+    from mxfp4_int8_m5_amd import sc_kernels
+    yield sc_kernels
+    sc_kernels.set_format(product_format(layout.DEFAULT))
+
+
+def test_unpack_quantized_matrix(S):
+    rng = np.random.default_rng(0)
+    n, k = 384, 2048
+    w = rng.standard_normal((n, k)) * 0.02 * rng.lognormal(0, 0.3, (1, k))
+    codes, bc, ws, qw = layout.quantize(w)
+    wq = host(S.unpack_i8(dev(codes), dev(bc), n, k, lazy=False))
+    assert np.array_equal(wq, qw)
+    assert np.array_equal(wq, layout.decode(codes, bc, n, k))
+
+
+@pytest.mark.parametrize("i", range(len(FORMATS)))
+def test_unpack_all_formats_random_codes(S, i):
+    fmt = FORMATS[i]
+    rng = np.random.default_rng(10 + i)
+    for n, k in ((256, 2048), (5, 128), (3, 64 if fmt.block * fmt.per_byte <= 64 else 128)):
+        if (k // fmt.block) % fmt.per_byte:
+            continue
+        codes, bc, ws, q = random_packed(rng, n, k, fmt)
+        wq = host(S.unpack_i8(dev(codes), dev(bc), n, k, lazy=False, fmt=product_format(fmt)))
+        assert np.array_equal(wq, q), (fmt, n, k)
+
+
+@pytest.mark.parametrize("m,k", [(200, 2048), (1, 128), (130, 6144), (7, 1000)])
+def test_act_quant(S, m, k):
+    rng = np.random.default_rng(m)
+    bits, x = llm_acts(rng, m, k)
+    if m > 3:
+        bits[3] = 0
+        x[3] = 0
+    xq, xs = S.act_quant(dev(bits))
+    rq, rs = linear.act_quant(x, S.pad_rows(m))
+    assert xq.shape[0] == S.pad_rows(m)
+    assert np.array_equal(host(xq), rq) and np.array_equal(host(xs), rs)
+    assert not host(xq)[m:].any() and not host(xs)[m:].any()
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 2048), (200, 384, 2048), (512, 2048, 1024), (64, 64, 128), (1, 4, 128),
+                                   (1024, 512, 256), (300, 260, 384)])
+def test_int32_gemm_exact(S, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    xq[0] = 127
+    ref = linear.int_gemm(xq, q)
+    a1 = host(S.mm_i8_i32(dev(xq), dev(q)))
+    assert np.array_equal(a1, ref), "INT8-weights GEMM"
+    packed = S.unpack_i8(dev(codes), dev(bc), n, k, lazy=True)
+    a2 = host(S.mm_i8_i32(dev(xq), packed))
+    assert np.array_equal(a2, ref), "fused-unpack GEMM"
+
+
+@pytest.mark.parametrize("i", range(1, len(FORMATS)))
+def test_int32_gemm_other_formats(S, i):
+    fmt = FORMATS[i]
+    rng = np.random.default_rng(40 + i)
+    m, n, k = 128, 256, 2048
+    codes, bc, ws, q = random_packed(rng, n, k, fmt)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    S.set_format(product_format(fmt))
+    acc = host(S.mm_i8_i32(dev(xq), S.unpack_i8(dev(codes), dev(bc), n, k)))
+    S.set_format(product_format(layout.DEFAULT))
+    assert np.array_equal(acc, linear.int_gemm(xq, q))
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 512, 1024), (128, 256, 2048), (2048, 2048, 256), (200, 136, 128)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_epilogues(S, m, n, k, packed):
+    """EPI 1/2/3 equal the INT32 GEMM + the reference formulas bit for bit (e2e/test_sc_kernels.py:121-142)."""
+    rng = np.random.default_rng(m * 7 + n)
+    codes, bc, _, q = random_packed(rng, n, k)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    xs = (np.abs(rng.standard_normal(m)) * 1e-3).astype(F32)
+    ws = (np.abs(rng.standard_normal(n)) * 1e-4).astype(F32)
+    res = bf16.to_bits(rng.standard_normal((m, n)).astype(F32))
+    acc = linear.int_gemm(xq, q)
+    wq = S.unpack_i8(dev(codes), dev(bc), n, k, lazy=packed)
+    y1 = host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 1, torch.bfloat16))
+    assert np.array_equal(y1, linear.epilogue(acc, xs, ws, 1))
+    y2 = host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 2, torch.bfloat16, res=dev(res)))
+    assert np.array_equal(y2, linear.epilogue(acc, xs, ws, 2, res))
+    perm = linear.interleave_gate_up(n // 2)
+    assert np.array_equal(perm, S.interleave_gate_up(n // 2))
+    if packed:
+        wq3 = S.unpack_i8(dev(codes.reshape(n, -1)[perm].reshape(-1)), dev(bc[perm]), n, k, lazy=True)
+    else:
+        wq3 = dev(q[perm])
+    y3 = host(S.mm_epi(dev(xq), wq3, dev(xs), dev(ws[perm]), 3, torch.bfloat16))
+    y = linear.scale_out(acc, xs, ws)
+    assert np.array_equal(y3, linear.swiglu(y[:, :n // 2], y[:, n // 2:]))
+
+
+def test_config0_dense_layer(S):
+    """BASELINE config 0: N = K = 2048, M = 512, SC-MXFP4-quantized N(0, 0.02) weights with outlier columns, bf16
+    activations with outlier channels; INT32 accumulators bit-exact, bf16 output within 1e-2 of the float path."""
+    rng = np.random.default_rng(0)
+    n = k = 2048
+    m = 512
+    w = llm_weights(rng, n, k)
+    codes, bc, ws, q = layout.quantize(w)
+    bits, x = llm_acts(rng, m, k)
+    xq_ref, xs_ref = linear.act_quant(x)
+    acc_ref = linear.int_gemm(xq_ref, q)
+    xq, xs = S.act_quant(dev(bits), Mp=m)
+    assert np.array_equal(host(xq), xq_ref) and np.array_equal(host(xs), xs_ref)
+    wq = S.unpack_i8(dev(codes), dev(bc), n, k)
+    assert np.array_equal(host(S.mm_i8_i32(xq, wq)), acc_ref)
+    y = host(S.linear_w4a8(dev(bits), dev(codes), dev(bc), dev(ws), n))
+    assert np.array_equal(y, linear.epilogue(acc_ref, xs_ref, ws, 1))
+    ref = linear.float_reference(x, q, ws)
+    assert linear.rel_fro(bf16.from_bits(y), ref) < 1e-2          # tolerance stated by the north star
+    assert linear.rel_fro(bf16.from_bits(y), x.astype(np.float64) @ w.T) < 0.2   # and it is the layer it claims to be
+
+
+@pytest.mark.parametrize("name,n,k", [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048),
+                                      ("down", 2048, 6144)])
+def test_config1_full_size_m2048(S, name, n, k):
+    """BASELINE config 1 at M = 2048: all INT32 accumulators against the float64 integer GEMM, the bf16 epilogue
+    bit for bit, and column-linearity of the accumulators (acc(x1 + x2) = acc(x1) + acc(x2))."""
+    rng = np.random.default_rng(n + k)
+    m = 2048
+    codes, bc, ws, q = random_packed(rng, n, k)
+    bits, x = llm_acts(rng, m, k)
+    xq_ref, xs_ref = linear.act_quant(x)
+    acc_ref = linear.int_gemm(xq_ref, q)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    xq, xs = S.act_quant(dev(bits), Mp=m)
+    wq = S.unpack_i8(dc, db, n, k)
+    acc = host(S.mm_i8_i32(xq, wq))
+    assert np.array_equal(acc, acc_ref)
+    y = host(S.linear_w4a8(dev(bits), dc, db, dw, n))
+    assert np.array_equal(y, linear.epilogue(acc_ref, xs_ref, ws, 1))
+    a = rng.integers(-60, 61, (256, k)).astype(np.int8)
+    b = rng.integers(-60, 61, (256, k)).astype(np.int8)
+    s = host(S.mm_i8_i32(dev(a), wq)) + host(S.mm_i8_i32(dev(b), wq))
+    assert np.array_equal(host(S.mm_i8_i32(dev((a + b).astype(np.int8)), wq)), s)
+
+
+def test_bad_arguments_raise(S):
+    xq = torch.zeros((4, 100), dtype=torch.int8, device="cuda")
+    wq = torch.zeros((8, 100), dtype=torch.int8, device="cuda")
+    with pytest.raises(ValueError):
+        S.mm_i8_i32(xq, wq)                      # K not a multiple of 128
+    with pytest.raises(ValueError):
+        S.act_quant(torch.zeros((4, 64), dtype=torch.bfloat16))   # CPU tensor

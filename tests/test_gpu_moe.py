@@ -1,0 +1,173 @@
+"""Mixture-of-experts parity on the GPU through the C ABI: token sort contract, grouped GEMM against per-expert
+float64 integer GEMMs (uneven segments, empty experts), epilogues, the two-pass variant, the weighted combine.
+Mirrors e2e/sc_moe.py:209-244 and e2e/test_sc_kernels.py:190-205."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bf16, layout, linear, moe
+from tests.util import FORMATS, dev, host, product_format, random_packed
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def M():
+    from mxfp4_int8_m5_amd import sc_moe
+    return sc_moe
+
+
+def skewed_routing(rng, tokens, experts, topk):
+    """softmax(N(0,1) logits + N(0,1.5) expert bias) -> top-k experts and renormalised bf16 scores."""
+    logits = rng.standard_normal((tokens, experts)) + rng.standard_normal(experts) * 1.5
+    p = np.exp(logits - logits.max(1, keepdims=True))
+    p /= p.sum(1, keepdims=True)
+    inds = np.argsort(-p, axis=1)[:, :topk]
+    sc = np.take_along_axis(p, inds, 1)
+    sc /= sc.sum(1, keepdims=True)
+    return inds.astype(np.int32), bf16.to_bits(sc.astype(F32))
+
+
+@pytest.mark.parametrize("m,topk,e,tm", [(75, 8, 8, 64), (4096, 8, 64, 128), (2048, 9, 257, 64), (1, 8, 64, 64),
+                                         (300, 1, 1024, 128)])
+def test_route_sort_contract(M, m, topk, e, tm):
+    rng = np.random.default_rng(m + e)
+    inds, _ = skewed_routing(rng, m, e, topk)
+    if e == 8:
+        inds[inds == 3] = 2          # an empty expert
+    pos, tok, es, off, ts, mt = M.route_sort(dev(inds), e, tm)
+    moe.check_route_sort(inds, e, tm, host(pos), host(tok), host(es), host(off), host(ts))
+    assert mt == -(-m * topk // tm) + e
+    ro = moe.route_sort(inds, e, tm)
+    assert np.array_equal(host(off), ro[3]) and np.array_equal(host(ts), ro[4]) and np.array_equal(host(es), ro[2])
+    o2, t2, mt2 = M.segments(es, e, tm)
+    assert np.array_equal(host(o2), ro[3]) and np.array_equal(host(t2), ro[4]) and mt2 == mt
+
+
+@pytest.mark.parametrize("tm", [64, 128])
+def test_grouped_gemm_uneven_segments(M, tm):
+    """8 experts, 600 rows, experts 3 and 7 empty (e2e/sc_moe.py:213-215): INT32 exact, EPI 1 and 3 bit-exact,
+    two-pass variant identical."""
+    rng = np.random.default_rng(0)
+    e, n, k, r = 8, 256, 512, 600
+    ex = np.sort(rng.choice(e - 1, r, p=np.r_[0.4, np.full(e - 2, 0.6 / (e - 2))])).astype(np.int32)
+    ex[ex == 3] = 2
+    packs = [layout.quantize(rng.standard_normal((n, k)) * 0.02) for _ in range(e)]
+    codes, bc, ws = (np.stack([p[i] for p in packs]) for i in range(3))
+    wq = np.stack([p[3] for p in packs])
+    xq = rng.integers(-127, 128, (r, k)).astype(np.int8)
+    xs = (np.abs(rng.standard_normal(r)) * 1e-2).astype(F32)
+    ref = moe.moe_int_gemm(xq, ex, wq)
+    off, tstart, mt = M.segments(dev(ex), e, tm)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    acc = host(M.moe_mm(dev(xq), r, dc, db, dw, off, tstart, mt, n, 0, tile=(tm, 64, 4)))
+    assert np.array_equal(acc, ref)
+    y1 = host(M.moe_mm(dev(xq), r, dc, db, dw, off, tstart, mt, n, 1, dev(xs), tile=(tm, 64, 4)))
+    assert np.array_equal(y1, moe.moe_epilogue(ref, xs, ws, ex, 1))
+    y3 = host(M.moe_mm(dev(xq), r, dc, db, dw, off, tstart, mt, n, 3, dev(xs), tile=(tm, 64, 4)))
+    assert np.array_equal(y3, moe.moe_epilogue(ref, xs, ws, ex, 3))
+    wq8 = M.unpack_experts(dc, db, n, k)
+    assert np.array_equal(host(wq8), wq.reshape(e * n, k))
+    acc2 = host(M.moe_mm_i8(dev(xq), r, wq8, dw, off, tstart, mt, n, 0, tile=(tm, 64, 4)))
+    assert np.array_equal(acc2, ref)
+
+
+@pytest.mark.parametrize("i", range(len(FORMATS)))
+def test_grouped_gemm_formats(M, i):
+    """Two experts with the same random-code weights, uneven segments (e2e/test_formats.py:46-52)."""
+    fmt = FORMATS[i]
+    rng = np.random.default_rng(80 + i)
+    n, k, m = 256, 2048, 128
+    codes, bc, ws, q = random_packed(rng, n, k, fmt)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    ex = np.sort(rng.integers(0, 2, m)).astype(np.int32)
+    off, tstart, mt = M.segments(dev(ex), 2, 64)
+    acc = host(M.moe_mm(dev(xq), m, dev(np.stack([codes, codes])), dev(np.stack([bc, bc])), dev(np.stack([ws, ws])),
+                        off, tstart, mt, n, 0, fmt=product_format(fmt)))
+    assert np.array_equal(acc, linear.int_gemm(xq, q))
+
+
+def test_moe_block_with_fused_gather_and_combine(M):
+    """A whole expert block at reduced width: route_sort -> grouped gate|up GEMM with SwiGLU reading token rows through
+    `gather` -> act_quant -> grouped down GEMM -> weighted combine; every stage against the oracle, and the result
+    independent of the order inside the segments."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    rng = np.random.default_rng(3)
+    tokens, e, topk, d, f, tm = 300, 16, 4, 256, 128, 64
+    inds, scores = skewed_routing(rng, tokens, e, topk)
+    gu = [random_packed(rng, 2 * f, d) for _ in range(e)]
+    dn = [random_packed(rng, d, f) for _ in range(e)]
+    perm = linear.interleave_gate_up(f)
+    gc = np.stack([p[0].reshape(2 * f, -1)[perm].reshape(-1) for p in gu])
+    gb = np.stack([p[1][perm] for p in gu])
+    gw = np.stack([p[2][perm] for p in gu])
+    gq = np.stack([p[3][perm] for p in gu])
+    dcodes, dbc, dws, dq = (np.stack([p[i] for p in dn]) for i in range(4))
+    xb = bf16.to_bits(rng.standard_normal((tokens, d)).astype(F32))
+    res = bf16.to_bits(rng.standard_normal((tokens, d)).astype(F32))
+    # GPU
+    xq, xs = S.act_quant(dev(xb), Mp=tokens)
+    pos, tok, es, off, ts, mt = M.route_sort(dev(inds), e, tm)
+    r = tokens * topk
+    act = M.moe_mm(xq, r, dev(gc), dev(gb), dev(gw), off, ts, mt, 2 * f, 3, xs, tile=(tm, 64, 4), gather=tok)
+    aq, as_ = S.act_quant(act, Mp=r)
+    yd = M.moe_mm(aq, r, dev(dcodes), dev(dbc), dev(dws), off, ts, mt, d, 1, as_, tile=(tm, 64, 4))
+    h, _, _ = M.moe_combine(yd, pos, dev(scores), dev(res), None, None, tokens, quant=False)
+    # oracle, with the GPU's own permutation (the order inside a segment is free)
+    pos_h, tok_h, es_h = host(pos), host(tok)[:r], host(es)
+    moe.check_route_sort(inds, e, tm, pos_h, host(tok), es_h, host(off), host(ts))
+    rq, rs = linear.act_quant(bf16.from_bits(xb))
+    acc1 = moe.moe_int_gemm(rq[tok_h], es_h, gq)
+    act_ref = moe.moe_epilogue(acc1, rs[tok_h], gw, es_h, 3)
+    assert np.array_equal(host(act), act_ref)
+    aq_ref, as_ref = linear.act_quant(bf16.from_bits(act_ref))
+    yd_ref = moe.moe_epilogue(moe.moe_int_gemm(aq_ref, es_h, dq), as_ref, dws, es_h, 1)
+    assert np.array_equal(host(yd), yd_ref)
+    h_ref = moe.combine(yd_ref, pos_h, scores, res, tokens)
+    assert np.array_equal(host(h), h_ref)
+    # the same block from the oracle's stable sort gives the same residual stream
+    p2, t2, e2, *_ = moe.route_sort(inds, e, tm)
+    a2 = moe.moe_epilogue(moe.moe_int_gemm(rq[t2[:r]], e2, gq), rs[t2[:r]], gw, e2, 3)
+    q2, s2 = linear.act_quant(bf16.from_bits(a2))
+    y2 = moe.moe_epilogue(moe.moe_int_gemm(q2, e2, dq), s2, dws, e2, 1)
+    assert np.array_equal(moe.combine(y2, p2, scores, res, tokens), h_ref)
+
+
+def test_combine_with_next_norm_and_split(M):
+    rng = np.random.default_rng(2)
+    m, mp, topk, k = 200, 256, 8, 2048
+    inds = np.stack([rng.permutation(64)[:topk] for _ in range(m)]).astype(np.int32)
+    pos, *_ = moe.route_sort(inds, 64, 64)
+    y = bf16.to_bits(rng.standard_normal((m * topk, k)).astype(F32))
+    sc = bf16.to_bits(np.abs(rng.standard_normal((m, topk))).astype(F32) * 0.2)
+    res = bf16.to_bits((rng.standard_normal((mp, k)) * 2).astype(F32))
+    nw = bf16.to_bits(rng.lognormal(0, 0.3, k).astype(F32))
+    h, xq, xs = M.moe_combine(dev(y), dev(pos), dev(sc), dev(res), dev(nw), 1e-5, m)
+    h_ref = moe.combine(y, pos, sc, res, m)
+    assert np.array_equal(host(h), h_ref)
+    rq, rs, _ = linear.rmsnorm_quant(h_ref, nw, 1e-5)
+    assert np.array_equal(host(xq), rq) and np.array_equal(host(xs), rs)
+    h2, _, _ = M.moe_combine_split(dev(y), dev(pos), dev(np.ascontiguousarray(sc[:, :-1])),
+                                   dev(np.ascontiguousarray(sc[:, -1])), dev(res), None, None, m)
+    assert np.array_equal(host(h2), h_ref)
+
+
+def test_config3_olmoe_shape_property(M):
+    """BASELINE config 3 at full size (64 experts, top-8, 4096 tokens, hidden 2048): the grouped INT32 accumulators
+    of the down projection (K = 1024) for every row against per-expert float64 GEMMs."""
+    rng = np.random.default_rng(33)
+    tokens, e, topk, d, f = 4096, 64, 8, 2048, 1024
+    inds, _ = skewed_routing(rng, tokens, e, topk)
+    codes1, bc1, ws1, q1 = random_packed(rng, d, f)
+    shift = rng.integers(0, e)
+    # per-expert weights: rows of one random matrix rolled by the expert index (cheap to build, all experts differ)
+    codes = np.stack([np.roll(codes1.reshape(d, -1), ex + shift, 0).reshape(-1) for ex in range(e)])
+    bc = np.stack([np.roll(bc1, ex + shift, 0) for ex in range(e)])
+    ws = np.stack([np.roll(ws1, ex + shift, 0) for ex in range(e)])
+    wq = np.stack([np.roll(q1, ex + shift, 0) for ex in range(e)])
+    r = tokens * topk
+    xq = rng.integers(-127, 128, (r, f)).astype(np.int8)
+    pos, tok, es, off, ts, mt = M.route_sort(dev(inds), e, 128)
+    acc = host(M.moe_mm(dev(xq), r, dev(codes), dev(bc), dev(ws), off, ts, mt, d, 0, tile=(128, 64, 4)))
+    assert np.array_equal(acc, moe.moe_int_gemm(xq, host(es), wq))
