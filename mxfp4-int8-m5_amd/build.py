@@ -10,7 +10,7 @@ LIB = os.path.join(HERE, "libscmx.so")
 SOURCES = ["api.hip", "gemm.hip", "gemv.hip", "rowops.hip"]
 # packed FP32 instructions are kept off (they have misbehaved on this hardware pool); no FMA contraction, so the
 # FP32 epilogues and norms round exactly like a plain IEEE evaluation
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wno-unused-command-line-argument",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-Wno-unused-command-line-argument",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

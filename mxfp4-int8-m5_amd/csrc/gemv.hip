@@ -70,7 +70,7 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
         __syncthreads();
         if (wave == 0) {
             const float tot = wave_sum(lane < (K / 4 + 63) / 64 ? red[lane] : 0.0f);
-            if (lane == 0) red[64] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, float(K)), a.eps)));
+            if (lane == 0) red[64] = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(tot, float(K)), a.eps)));
         }
         __syncthreads();
         inv = red[64];

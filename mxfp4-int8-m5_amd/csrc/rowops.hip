@@ -32,7 +32,7 @@ __device__ float block_inv_rms(const uint16_t* xr, int K, float eps, float* red)
     __syncthreads();
     if (wave == 0) {
         const float tot = wave_sum(lane < groups ? red[lane] : 0.0f);
-        if (lane == 0) red[64] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, float(K)), eps)));
+        if (lane == 0) red[64] = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(tot, float(K)), eps)));
     }
     __syncthreads();
     const float inv = red[64];
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
         uint16_t* o = out + (size_t(hh) * L + row) * d + per * lane;
         if (g < hq + hk) {
             ss = wave_sum(ss);
-            const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
+            const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
             const uint16_t* w = g < hq ? qn : kn;
             for (int i = 0; i < per; ++i)
                 o[i] = f32_to_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
