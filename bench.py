@@ -1,0 +1,226 @@
+"""Benchmark of the SC-MXFP4 W4A8 hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass of the dense W4A8 linear (activation-quantization prologue + fused-unpack INT8-MFMA GEMM + bf16
+epilogue, through the C ABI entry scmx_linear_w4a8) over the four Qwen3-1.7B-shaped layers at M = 2048 tokens
+(BASELINE config 1): qkv 4096x2048, o_proj 2048x2048, gate_up 12288x2048, down 2048x6144.  Inputs are seeded
+synthetic tensors already resident in HBM; weight sets rotate so that consecutive steps do not reuse cached weights.
+`value` is INT8 TOPS = 2*M*N*K summed over the layers / time.  The same run also reports the decode GEMV's achieved
+HBM GB/s (config 2) and a CPU baseline (the numpy oracle on the host cores).  Prints ONE JSON line.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0        # MI355X dense INT8 MFMA, published
+PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E, published
+M_TOKENS = 2048
+LAYERS = [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]
+DECODE = LAYERS + [("lm_head", 151936, 2048)]
+
+
+def packed_random(rng, n, k):
+    """Random SC-MXFP4 codes: statistically the quantized N(0, 0.02) matrix's storage (all 16 codes and 4 shifts occur);
+    throughput does not depend on the values."""
+    codes = rng.integers(0, 2 ** 32, n * k // 8, dtype=np.uint64).astype(np.uint32)
+    bc = rng.integers(0, 256, (n, k // 128), dtype=np.uint16).astype(np.uint8)
+    ws = np.exp2(rng.integers(-12, -6, n)).astype(np.float32)
+    return codes, bc, ws
+
+
+def acts(rng, m, k):
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[:, rng.choice(k, max(1, round(0.01 * k)), replace=False)] *= 20
+    return x
+
+
+def cpu_baseline(budget_s=12.0):
+    """The oracle's path (numpy): per-token INT8 quantization, float64-BLAS integer GEMM, FP32 scaling, bf16 rounding,
+    for the four layers at M = 2048 with pre-decoded INT8 weights; repeated until the time budget is used."""
+    from oracle import bf16, linear
+    rng = np.random.default_rng(1)
+    work = []
+    for _, n, k in LAYERS:
+        wq = rng.integers(-96, 97, (n, k)).astype(np.int8)
+        ws = np.exp2(rng.integers(-12, -6, n)).astype(np.float32)
+        work.append((bf16.rnd(acts(rng, M_TOKENS, k)), wq, ws))
+    ops = sum(2.0 * M_TOKENS * n * k for _, n, k in LAYERS)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        for x, wq, ws in work:
+            xq, xs = linear.act_quant(x)
+            linear.epilogue(linear.int_gemm(xq, wq), xs, ws, 1)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 50:
+            break
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        threads = os.cpu_count()
+    return {"value": round(ops * reps / el / 1e12, 4), "unit": "TOPS", "cores": int(threads), "kind": "port",
+            "sample": f"{reps} pass(es) of the 4 layers at M={M_TOKENS} (act quant + float64 BLAS integer GEMM + bf16 "
+                      f"epilogue, INT8 weights pre-decoded), {el:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV leg")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mxfp4_int8_m5_amd as pkg
+    lib = pkg._lib.load()
+    fmt = pkg.sc_format.DEFAULT.c_struct()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream()
+    sp = C.c_void_p(stream.cuda_stream)
+    rng = np.random.default_rng(1)
+
+    def up(arr):
+        arr = np.ascontiguousarray(arr)
+        if arr.dtype == np.uint32:
+            arr = arr.view(np.int32)
+        return torch.from_numpy(arr).to(dev)
+
+    # ---- prefill: weight sets rotate (> 256 MB in total, beyond the last-level cache) --------------------------
+    set_bytes = sum(n * k // 2 + n * k // 128 + 4 * n for _, n, k in LAYERS)
+    n_sets = max(2, -(-300 * 2 ** 20 // set_bytes))
+    sets = []
+    for _ in range(n_sets):
+        sets.append([tuple(up(t) for t in packed_random(rng, n, k)) for _, n, k in LAYERS])
+    xs_in = {k: up(acts(rng, M_TOKENS, k)).to(torch.bfloat16) for k in sorted({k for _, _, k in LAYERS})}
+    outs = [torch.empty((M_TOKENS, n), dtype=torch.bfloat16, device=dev) for _, n, _ in LAYERS]
+    ws_bytes = max(lib.scmx_linear_w4a8_workspace(M_TOKENS, k) for _, _, k in LAYERS)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(lib.scmx_last_error().decode())
+
+    calls = []
+    for s in sets:
+        step = []
+        for (name, n, k), (codes, bc, ws), out in zip(LAYERS, s, outs):
+            step.append((C.byref(fmt), xs_in[k].data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(), None,
+                         out.data_ptr(), 1, M_TOKENS, n, k, workspace.data_ptr(), ws_bytes, sp))
+        calls.append(step)
+
+    def run_step(i):
+        for args in calls[i % n_sets]:
+            check(lib.scmx_linear_w4a8(*args))
+
+    for i in range(a.warmup):
+        run_step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(a.steps):
+        run_step(i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms_step = e0.elapsed_time(e1) / a.steps
+    ops_step = sum(2.0 * M_TOKENS * n * k for _, n, k in LAYERS)
+    tops = ops_step / (ms_step * 1e-3) / 1e12
+
+    # ---- roofline of the dominant kernel (the fused-unpack GEMM alone, activations pre-quantized) -------------------
+    per_shape = {}
+    tot_ops = tot_ms = 0.0
+    reps = max(20, a.steps // 2)
+    for li, (name, n, k) in enumerate(LAYERS):
+        xq = torch.empty((M_TOKENS, k), dtype=torch.int8, device=dev)
+        xs = torch.empty(M_TOKENS, dtype=torch.float32, device=dev)
+        check(lib.scmx_act_quant(xs_in[k].data_ptr(), xq.data_ptr(), xs.data_ptr(), M_TOKENS, M_TOKENS, k, sp))
+        argl = []
+        for s in sets:
+            codes, bc, ws = s[li]
+            argl.append((C.byref(fmt), xq.data_ptr(), xs.data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(), None,
+                         outs[li].data_ptr(), 1, M_TOKENS, n, k, sp))
+        for i in range(5):
+            check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for i in range(reps):
+            check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        ops = 2.0 * M_TOKENS * n * k
+        per_shape[name] = {"us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
+                           "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
+        tot_ops += ops
+        tot_ms += ms
+    achieved = tot_ops / tot_ms / 1e9
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None, "kernel": "scmx::gemm_kernel (mm_w4a8)",
+                "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their average launch "
+                        "durations, activations pre-quantized", "per_shape": per_shape}
+
+    # ---- decode GEMV: achieved HBM GB/s, weights rotating beyond the cache -----------------------------------------
+    decode = {}
+    if not a.no_decode:
+        del sets, calls
+        torch.cuda.empty_cache()
+        for name, n, k in DECODE:
+            bytes_call = n * k * (0.5 + 1.0 / 128) + 4 * n + 2 * k + 2 * n      # packed codes + 2-bit block codes + row
+            copies = max(2, -(-320 * 2 ** 20 // int(bytes_call)))              # scales + bf16 in / out
+            copies = min(copies, 160)
+            wsets = [tuple(up(t) for t in packed_random(rng, n, k)) for _ in range(copies)]
+            for batch in (1, 4):
+                x = up(acts(rng, batch, k)).to(torch.bfloat16)
+                out = torch.empty((batch, n), dtype=torch.bfloat16, device=dev)
+                argl = [(C.byref(fmt), x.data_ptr(), None, c.data_ptr(), b.data_ptr(), w.data_ptr(), None, out.data_ptr(),
+                         1, 1, None, C.c_float(0.0), batch, n, k, None, 0, 0, -1, sp) for c, b, w in wsets]
+                for i in range(copies):
+                    check(lib.scmx_gemv(*argl[i]))
+                torch.cuda.synchronize()
+                reps_d = max(copies, 100)
+                e0.record(stream)
+                for i in range(reps_d):
+                    check(lib.scmx_gemv(*argl[i % copies]))
+                e1.record(stream)
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) / reps_d * 1e3
+                bts = n * k * (0.5 + 1.0 / 128) + 4 * n + batch * (2 * k + 2 * n)
+                decode[f"{name}_b{batch}"] = {"us": round(us, 2), "gbps": round(bts / us / 1e3, 1),
+                                              "pct_hbm": round(bts / us / 1e3 / PEAK_HBM_GBPS * 100, 1)}
+            del wsets
+            torch.cuda.empty_cache()
+
+    result = {
+        "metric": "INT8 TOPS, W4A8 prefill GEMM M=2048 (Qwen3-1.7B layer shapes), 1 GPU; decode GEMV GB/s alongside",
+        "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1] at M=2048: SC-MXFP4 W4A8 linear (act-quant prologue + fused-unpack "
+                               "INT8 MFMA GEMM + bf16 epilogue) over qkv 4096x2048, o_proj 2048x2048, gate_up 12288x2048, "
+                               "down 2048x6144", "tokens": M_TOKENS, "weight_sets_rotated": n_sets},
+        "pct_int8_peak": round(tops / PEAK_INT8_TOPS * 100, 2),
+        "roofline": roofline,
+        "decode": decode,
+    }
+    if not a.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
