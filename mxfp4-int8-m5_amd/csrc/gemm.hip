@@ -8,6 +8,8 @@
 // of 4 consecutive output columns n of one token row m, which is the unit every epilogue works on.
 // LDS is double buffered: global loads for step i+1 are issued before the MFMAs of step i, decoded and stored
 // after them, with one barrier per step.
+#include <type_traits>
+
 #include "scmx_common.h"
 
 namespace scmx {
@@ -31,24 +33,28 @@ struct GemmArgs {
     DevFormat fmt;
 };
 
-constexpr int PAD = 16;  // LDS row padding in bytes: consecutive rows start 4 banks apart modulo 64
-
 enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2 };
+
+constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
 
 template <int BM, int BN, int BK, int WGM, int WGN, int BMODE>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
     constexpr int NT = WGM * WGN * 64;
-    constexpr int RS = BK + PAD;             // LDS row stride in bytes
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int MI = WTM / 32, NI = WTN / 32;
-    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "tile must be whole 32x32x32 MFMAs");
-    constexpr int A_CHUNKS = BM * BK / 16;   // 16-byte pieces of the activation tile
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && (BK == 64 || BK == 128), "tile must be whole 32x32x32 MFMAs");
+    constexpr int CPR = BK / 16;             // 16-byte chunks per LDS row
+    constexpr int RPB = 256 / BK;            // rows per 256 bytes, i.e. per sweep of the 64 LDS banks
+    constexpr int A_CHUNKS = BM * CPR;       // 16-byte pieces of the activation tile
     constexpr int A_PER = (A_CHUNKS + NT - 1) / NT;
-    constexpr int B_CHUNKS = BMODE == B_INT8 ? BN * BK / 16 : BN * BK / 32;   // 16 bytes of INT8 or of codes
+    constexpr int B_CHUNKS = BMODE == B_INT8 ? BN * CPR : BN * BK / 32;   // 16 bytes of INT8 or of codes
     constexpr int B_PER = (B_CHUNKS + NT - 1) / NT;
+    constexpr int STAGE = (BM + BN) * BK;    // bytes per stage: BM activation rows then BN weight rows
 
-    __shared__ __attribute__((aligned(16))) int8_t sA[2][BM * RS];
-    __shared__ __attribute__((aligned(16))) int8_t sB[2][BN * RS];
+    // Rows are BK bytes with no padding; the 16-byte chunk c of row r sits at chunk c ^ ((r / RPB) % CPR), which
+    // spreads the 16 rows a b128 fragment read touches per pass over all 64 banks.
+    __shared__ __attribute__((aligned(16))) int8_t smem[NSTAGE * STAGE];
+    auto swz = [](int row, int chunk) { return row * BK + ((chunk ^ ((row / RPB) & (CPR - 1))) << 4); };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WGM, wn = wave / WGM;
@@ -86,23 +92,24 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < A_PER; ++j) {
         const int c = tid + j * NT;
-        const int row = c / (BK / 16), kc = c % (BK / 16);
+        const int row = c / CPR, kc = c % CPR;
         int gr = min(m0 + row, a.M - 1);
         if (a.gather) gr = a.gather[gr];
         a_src[j] = a.xq + size_t(gr) * K + kc * 16;
-        a_dst[j] = row * RS + kc * 16;
+        a_dst[j] = swz(row, kc);
     }
     const uint8_t* b_src[B_PER];
     const uint8_t* b_bc[B_PER];
-    int b_dst[B_PER], b_k[B_PER];
+    int b_dst[B_PER], b_dst2[B_PER], b_k[B_PER];
 #pragma unroll
     for (int j = 0; j < B_PER; ++j) {
         const int c = tid + j * NT;
         if (BMODE == B_INT8) {
-            const int row = c / (BK / 16), kc = c % (BK / 16);
+            const int row = c / CPR, kc = c % CPR;
             const int gn = min(n0 + row, a.N - 1);
             b_src[j] = reinterpret_cast<const uint8_t*>(a.wq) + (size_t(expert) * a.N + gn) * K + kc * 16;
-            b_dst[j] = row * RS + kc * 16;
+            b_dst[j] = BM * BK + swz(row, kc);
+            b_dst2[j] = 0;
             b_bc[j] = nullptr;
             b_k[j] = 0;
         } else {
@@ -110,63 +117,81 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
             const int gn = min(n0 + row, a.N - 1);
             b_src[j] = reinterpret_cast<const uint8_t*>(a.codes) + (size_t(expert) * a.N + gn) * (K / 2) + kb * 16;
             b_bc[j] = a.bcodes + (size_t(expert) * a.N + gn) * a.bc_row_bytes;
-            b_dst[j] = row * RS + kb * 32;
+            b_dst[j] = BM * BK + swz(row, 2 * kb);
+            b_dst2[j] = BM * BK + swz(row, 2 * kb + 1);
             b_k[j] = kb * 32;
         }
     }
 
-    u32x4 ra[A_PER], rb[B_PER];
-    uint32_t rbc[B_PER];
+    // Two register sets hold the global loads of two K steps in flight.
+    struct Staged {
+        u32x4 a[A_PER], b[B_PER];
+        uint32_t bc[B_PER];
+    };
+    Staged r0, r1;
 
-    auto load_global = [&](int k0) {
+    // Loads past the last K step re-read the last step (never consumed): every iteration issues the same loads, so
+    // the wait before a register set is used covers exactly that set and not the younger one.
+    auto load_global = [&](Staged& r, int k0) {
+        k0 = min(k0, K - BK);
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
             if (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS)
-                ra[j] = *reinterpret_cast<const u32x4*>(a_src[j] + k0);
+                r.a[j] = *reinterpret_cast<const u32x4*>(a_src[j] + k0);
 #pragma unroll
         for (int j = 0; j < B_PER; ++j)
             if (B_CHUNKS % NT == 0 || tid + j * NT < B_CHUNKS) {
                 if (BMODE == B_INT8) {
-                    rb[j] = *reinterpret_cast<const u32x4*>(b_src[j] + k0);
+                    r.b[j] = *reinterpret_cast<const u32x4*>(b_src[j] + k0);
                 } else {
-                    rb[j] = *reinterpret_cast<const u32x4*>(b_src[j] + (k0 >> 1));
-                    if (BMODE == B_PACKED_DEFAULT) {   // 32-blocks, 2-bit codes: 4 blocks per byte
-                        const uint32_t blk = uint32_t(k0 + b_k[j]) >> 5;
-                        rbc[j] = (uint32_t(b_bc[j][blk >> 2]) >> (2 * (blk & 3))) & 3u;
-                    }
+                    r.b[j] = *reinterpret_cast<const u32x4*>(b_src[j] + (k0 >> 1));
+                    if (BMODE == B_PACKED_DEFAULT)   // 32-blocks, 2-bit codes, 4 blocks per byte: keep the raw byte
+                        r.bc[j] = b_bc[j][uint32_t(k0 + b_k[j]) >> 7];
                 }
             }
     };
 
-    auto store_lds = [&](int buf, int k0) {
+    // Staging work of one K step, cut into NKK slices so that it can be issued in the shadow of the MFMAs of the
+    // step being multiplied: slice q writes the activation chunks j with j % NKK == q and decodes the weight code
+    // words w with w * NKK / 4 == q; the last slice writes the decoded weights.
+    constexpr int NKK = BK / 32;
+    auto stage_slice = [&](const Staged& r, int8_t* st, int k0, int q, uint32_t (&o)[B_PER][8]) {
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
-            if (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS)
-                *reinterpret_cast<u32x4*>(&sA[buf][a_dst[j]]) = ra[j];
+            if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS))
+                *reinterpret_cast<u32x4*>(st + a_dst[j]) = r.a[j];
 #pragma unroll
         for (int j = 0; j < B_PER; ++j)
             if (B_CHUNKS % NT == 0 || tid + j * NT < B_CHUNKS) {
                 if (BMODE == B_INT8) {
-                    *reinterpret_cast<u32x4*>(&sB[buf][b_dst[j]]) = rb[j];
+                    if (q == 0) *reinterpret_cast<u32x4*>(st + b_dst[j]) = r.b[j];
                 } else {
-                    uint32_t o[8];
-                    if (BMODE == B_PACKED_DEFAULT) {
-                        const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, rbc[j]);
 #pragma unroll
-                        for (int w = 0; w < 4; ++w) decode_word(rb[j][w], t, o[2 * w], o[2 * w + 1]);
-                    } else {
-#pragma unroll
-                        for (int w = 0; w < 4; ++w) {
+                    for (int w = 0; w < 4; ++w) {
+                        if (w * NKK / 4 != q) continue;
+                        if (BMODE == B_PACKED_DEFAULT) {
+                            const uint32_t blk = uint32_t(k0 + b_k[j]) >> 5;
+                            const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, (r.bc[j] >> (2 * (blk & 3))) & 3u);
+                            decode_word(r.b[j][w], t, o[j][2 * w], o[j][2 * w + 1]);
+                        } else {
                             const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> a.fmt.block_log2;
                             const uint32_t bc = block_code(b_bc[j], blk, a.fmt.bc_bits);
                             const BlockLut t = scaled_lut_mul(a.fmt.lut_lo, a.fmt.lut_hi, mult_of(a.fmt, bc));
-                            decode_word(rb[j][w], t, o[2 * w], o[2 * w + 1]);
+                            decode_word(r.b[j][w], t, o[j][2 * w], o[j][2 * w + 1]);
                         }
                     }
-                    *reinterpret_cast<u32x4*>(&sB[buf][b_dst[j]]) = u32x4{o[0], o[1], o[2], o[3]};
-                    *reinterpret_cast<u32x4*>(&sB[buf][b_dst[j] + 16]) = u32x4{o[4], o[5], o[6], o[7]};
+                    if (q == NKK - 1) {
+                        *reinterpret_cast<u32x4*>(st + b_dst[j]) = u32x4{o[j][0], o[j][1], o[j][2], o[j][3]};
+                        *reinterpret_cast<u32x4*>(st + b_dst2[j]) = u32x4{o[j][4], o[j][5], o[j][6], o[j][7]};
+                    }
                 }
             }
+    };
+    auto store_lds = [&](const Staged& r, int stage, int k0) {
+        k0 = min(k0, K - BK);
+        uint32_t o[B_PER][8];
+#pragma unroll
+        for (int q = 0; q < NKK; ++q) stage_slice(r, smem + stage * STAGE, k0, q, o);
     };
 
     v16i acc[MI][NI];
@@ -177,93 +202,196 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    // fragment addresses: lane l supplies row l % 32 and the 16 k-bytes of half l / 32 of a 32-wide k slice
-    const int frag_off = (lane & 31) * RS + (lane >> 5) * 16;
-    const int a_frag = (wm * WTM) * RS + frag_off;
-    const int b_frag = (wn * WTN) * RS + frag_off;
+    // fragment addresses: lane l supplies row l % 32 and the 16 k-bytes of half l / 32 of a 32-wide k slice; tile
+    // origins are multiples of 32 rows, so the swizzle term depends on the lane only
+    const int lr = lane & 31, half = lane >> 5;
+    const int sw = (lr / RPB) & (CPR - 1);
+    int koff[NKK];
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) koff[kk] = ((2 * kk + half) ^ sw) << 4;
+    const int a_frag = (wm * WTM + lr) * BK;
+    const int b_frag = BM * BK + (wn * WTN + lr) * BK;
 
-    auto mma = [&](int buf) {
+    // Pipeline.  Iteration kt: barrier; multiply step kt out of its LDS stage while the register set holding step
+    // kt+2 is decoded and written into its stage, one slice per 32-wide k slice of MFMAs; then reissue that set's
+    // global loads for step kt+4.  A stage is rewritten two barriers after its last read and read two barriers after
+    // it was written; global loads have two iterations to land.
+    const int KT = K / BK;
+    load_global(r0, 0);
+    load_global(r1, BK);
+    store_lds(r0, 0, 0);
+    store_lds(r1, 1, BK);
+    load_global(r0, 2 * BK);
+    load_global(r1, 3 * BK);
+    int rd = 0;   // stage of step kt
+    auto load_frags = [&](const int8_t* src, int kk, v4i (&fa)[MI], v4i (&fb)[NI]) {
 #pragma unroll
-        for (int kk = 0; kk < BK / 32; ++kk) {
-            v4i fa[MI], fb[NI];
+        for (int i = 0; i < MI; ++i) fa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
-                fa[i] = *reinterpret_cast<const v4i*>(&sA[buf][a_frag + i * 32 * RS + kk * 32]);
+        for (int j = 0; j < NI; ++j) fb[j] = *reinterpret_cast<const v4i*>(src + b_frag + j * 32 * BK + koff[kk]);
+    };
+    auto iteration = [&](Staged& r, int kt) {
+        __syncthreads();
+        const int wr = rd == 0 ? NSTAGE - 1 : rd - 1;   // (kt + 2) % 3
+        const int8_t* src = smem + rd * STAGE;
+        int8_t* dst = smem + wr * STAGE;
+        const int k2 = min((kt + 2) * BK, K - BK);      // past the end: rewrites a stage nobody reads again
+        uint32_t o[B_PER][8];
+        v4i fa[2][MI], fb[2][NI];
+        load_frags(src, 0, fa[0], fb[0]);
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
-                fb[j] = *reinterpret_cast<const v4i*>(&sB[buf][b_frag + j * 32 * RS + kk * 32]);
+        for (int kk = 0; kk < NKK; ++kk) {
+            if (kk + 1 < NKK) load_frags(src, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+            stage_slice(r, dst, k2, kk, o);
         }
+        load_global(r, (kt + 4) * BK);
+        rd = rd == NSTAGE - 1 ? 0 : rd + 1;
     };
-
-    const int KT = K / BK;
-    load_global(0);
-    store_lds(0, 0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) load_global((kt + 1) * BK);
-        mma(cur);
-        if (more) store_lds(cur ^ 1, (kt + 1) * BK);
-        __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        iteration(r0, kt);
+        iteration(r1, kt + 1);
     }
+    if (kt < KT) iteration(r0, kt);
 
-    // ---- epilogue: lane holds acc[i][j][4g + r] = (m = tile_m + i*32 + lane%32, n = tile_n + j*32 + 8g + 4(lane/32) + r)
-    const int epi = a.epi;
+    // ---- epilogue ---------------------------------------------------------------------------------------------
+    // Lane holds acc[i][j][4g + r] = (m = i*32 + lane%32, n = j*32 + 8g + 4(lane/32) + r) of its wave tile: 4 consecutive
+    // columns of one row, the unit every epilogue works on.  Results go through a per-wave LDS tile so that global
+    // stores are 16 bytes per lane over whole contiguous row segments.
     const int N = a.N;
     const float* ws = a.wscale + size_t(expert) * N;
+    __syncthreads();   // every wave is done reading the staging buffers
+    auto epilogue = [&](auto epi_tag) {
+    constexpr int epi = decltype(epi_tag)::value;
+    constexpr int esize = epi == SCMX_EPI_I32 ? 4 : 2;
+    constexpr int ocols = epi == SCMX_EPI_SWIGLU ? WTN / 2 : WTN;     // output columns of the wave tile
+    const int on = epi == SCMX_EPI_SWIGLU ? N / 2 : N;            // output row length
+    constexpr int rowb = ocols * esize;                                // bytes per tile row
+    constexpr int rsb = rowb + 16;                                     // padded LDS row stride
+    constexpr bool fits = WGM * WGN * WTM * rsb <= NSTAGE * STAGE;   // per-wave tiles reuse the staging LDS
+    int8_t* wtile = smem + (fits ? wave * (WTM * rsb) : 0);
+    const int wm0 = m0 + wm * WTM, wn0 = n0 + wn * WTN;            // wave tile origin (input column index)
+    const bool wide = fits && (size_t(on) * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 &&
+                      (epi != SCMX_EPI_RES || reinterpret_cast<uintptr_t>(a.res) % 16 == 0);
+
+    // all scale loads of the wave tile are issued together, ahead of the conversions that use them
+    float xsv[MI];
+    f32x4 wsv[NI][4];
+    if (epi != SCMX_EPI_I32) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int m = wm0 + i * 32 + lr;
+            xsv[i] = m < row_end ? a.xscale[a.gather ? a.gather[m] : m] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = wn0 + j * 32 + 8 * g + 4 * half;
+                wsv[j][g] = n < N ? *reinterpret_cast<const f32x4*>(ws + n) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+    }
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
-        const int m = m0 + wm * WTM + i * 32 + (lane & 31);
-        if (m >= row_end) continue;
-        float xs = 0.0f;
-        if (epi != SCMX_EPI_I32) xs = a.xscale[a.gather ? a.gather[m] : m];
+        const int row = i * 32 + lr;
+        const int m = wm0 + row;
+        const float xs = epi != SCMX_EPI_I32 ? xsv[i] : 0.0f;
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * (lane >> 5);
-                if (n >= N) continue;
+                const int col = j * 32 + 8 * g + 4 * half;
+                const int n = wn0 + col;
                 if (epi == SCMX_EPI_I32) {
-                    *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(a.out) + size_t(m) * N + n) =
-                        v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    const v4i v = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    if (wide)
+                        *reinterpret_cast<v4i*>(wtile + row * rsb + col * 4) = v;
+                    else if (m < row_end && n < N)
+                        *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(a.out) + size_t(m) * N + n) = v;
                     continue;
                 }
-                const f32x4 w4 = *reinterpret_cast<const f32x4*>(ws + n);
+                const f32x4 w4 = wsv[j][g];
                 float y[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     y[r] = __fmul_rn(__fmul_rn(float(acc[i][j][4 * g + r]), xs), w4[r]);
                 uint16_t* out = reinterpret_cast<uint16_t*>(a.out);
-                if (epi == SCMX_EPI_SCALE) {
-                    u32x2 o;
-                    o[0] = uint32_t(f32_to_bf16(y[0])) | (uint32_t(f32_to_bf16(y[1])) << 16);
-                    o[1] = uint32_t(f32_to_bf16(y[2])) | (uint32_t(f32_to_bf16(y[3])) << 16);
-                    *reinterpret_cast<u32x2*>(out + size_t(m) * N + n) = o;
-                } else if (epi == SCMX_EPI_RES) {
-                    const u32x2 rr = *reinterpret_cast<const u32x2*>(a.res + size_t(m) * N + n);
-                    uint16_t h[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float rv = __uint_as_float(r & 1 ? (rr[r >> 1] & 0xFFFF0000u) : (rr[r >> 1] << 16));
-                        h[r] = f32_to_bf16(__fadd_rn(rv, round_bf16(y[r])));
-                    }
-                    u32x2 o;
-                    o[0] = uint32_t(h[0]) | (uint32_t(h[1]) << 16);
-                    o[1] = uint32_t(h[2]) | (uint32_t(h[3]) << 16);
-                    *reinterpret_cast<u32x2*>(out + size_t(m) * N + n) = o;
-                } else {   // SwiGLU of (g, g, u, u)
+                if (epi == SCMX_EPI_SWIGLU) {   // (g, g, u, u) -> two outputs
                     const uint16_t s0 = swiglu_bf16(round_bf16(y[0]), round_bf16(y[2]));
                     const uint16_t s1 = swiglu_bf16(round_bf16(y[1]), round_bf16(y[3]));
-                    *reinterpret_cast<uint32_t*>(out + size_t(m) * (N / 2) + n / 2) = uint32_t(s0) | (uint32_t(s1) << 16);
+                    const uint32_t o = uint32_t(s0) | (uint32_t(s1) << 16);
+                    if (wide)
+                        *reinterpret_cast<uint32_t*>(wtile + row * rsb + col) = o;
+                    else if (m < row_end && n < N)
+                        *reinterpret_cast<uint32_t*>(out + size_t(m) * on + n / 2) = o;
+                    continue;
+                }
+                u32x2 o;
+                o[0] = uint32_t(f32_to_bf16(y[0])) | (uint32_t(f32_to_bf16(y[1])) << 16);
+                o[1] = uint32_t(f32_to_bf16(y[2])) | (uint32_t(f32_to_bf16(y[3])) << 16);
+                if (wide) {
+                    *reinterpret_cast<u32x2*>(wtile + row * rsb + col * 2) = o;   // the residual is added on the way out
+                } else if (m < row_end && n < N) {
+                    if (epi == SCMX_EPI_RES) {
+                        const u32x2 rr = *reinterpret_cast<const u32x2*>(a.res + size_t(m) * N + n);
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+                            const float lo = __fadd_rn(__uint_as_float(rr[r] << 16), __uint_as_float(o[r] << 16));
+                            const float hi = __fadd_rn(__uint_as_float(rr[r] & 0xFFFF0000u), __uint_as_float(o[r] & 0xFFFF0000u));
+                            o[r] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+                        }
+                    }
+                    *reinterpret_cast<u32x2*>(out + size_t(m) * N + n) = o;
                 }
             }
         }
+    }
+    if (!wide) return;
+    __builtin_amdgcn_wave_barrier();   // LDS operations of one wave complete in order: the tile is visible to its lanes
+
+    // read the tile back 16 bytes per lane, whole rows at a time, and store
+    constexpr int ppr = rowb / 16;                 // 16-byte pieces per tile row (2, 4, 8 or 16)
+    constexpr int epp = 16 / esize;                // output elements per piece
+    const int ocol0 = epi == SCMX_EPI_SWIGLU ? wn0 / 2 : wn0;
+    for (int p = lane; p < WTM * ppr; p += 64) {
+        const int row = p / ppr, pc = p % ppr;
+        const int m = wm0 + row, c = ocol0 + pc * epp;
+        if (m >= row_end || c >= on) continue;
+        u32x4 v = *reinterpret_cast<const u32x4*>(wtile + row * rsb + pc * 16);
+        int8_t* dst = reinterpret_cast<int8_t*>(a.out) + (size_t(m) * on + c) * esize;
+        if (epi == SCMX_EPI_RES) {
+            const bool full = c + epp <= on;
+            u32x4 rr = u32x4{0u, 0u, 0u, 0u};
+            if (full) {
+                rr = *reinterpret_cast<const u32x4*>(a.res + size_t(m) * on + c);
+            } else {
+                const u32x2 r2 = *reinterpret_cast<const u32x2*>(a.res + size_t(m) * on + c);
+                rr[0] = r2[0];
+                rr[1] = r2[1];
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float lo = __fadd_rn(__uint_as_float(rr[r] << 16), __uint_as_float(v[r] << 16));
+                const float hi = __fadd_rn(__uint_as_float(rr[r] & 0xFFFF0000u), __uint_as_float(v[r] & 0xFFFF0000u));
+                v[r] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+            }
+        }
+        if (c + epp <= on)
+            *reinterpret_cast<u32x4*>(dst) = v;
+        else   // the row ends inside this piece: rows are multiples of 4 elements, so exactly half of it is valid
+            *reinterpret_cast<u32x2*>(dst) = u32x2{v[0], v[1]};
+    }
+    };
+    switch (a.epi) {
+        case SCMX_EPI_I32: epilogue(std::integral_constant<int, SCMX_EPI_I32>{}); break;
+        case SCMX_EPI_SCALE: epilogue(std::integral_constant<int, SCMX_EPI_SCALE>{}); break;
+        case SCMX_EPI_RES: epilogue(std::integral_constant<int, SCMX_EPI_RES>{}); break;
+        default: epilogue(std::integral_constant<int, SCMX_EPI_SWIGLU>{}); break;
     }
 }
 
