@@ -102,14 +102,37 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
     return s;
 }
 
+// Wave sum with DPP adds (one VALU instruction per step): quad swaps, half-row and row mirrors, then the two row
+// broadcasts.  The total is valid in lane 63 only.
+__device__ __forceinline__ int wave_sum_to_lane63(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);    // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);    // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);   // row_half_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, false);   // row_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);   // row_bcast15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);   // row_bcast31 into rows 2 and 3
+    return v;
+}
+
+// Per-byte negation of INT8 bytes in -127..127.
+__device__ __forceinline__ uint32_t neg_i8x4(uint32_t x) {
+    const uint32_t n = ~x;
+    return ((n & 0x7F7F7F7Fu) + 0x01010101u) ^ (n & 0x80808080u);
+}
+
 template <int BATCH, int R, bool DEFAULT_FMT>
 __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     constexpr int NT = 256;
+    constexpr int NV = R * BATCH;
+    constexpr bool XSEL = DEFAULT_FMT && BATCH == 1;   // signs applied to the activations instead of the weights
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
-    int8_t* sx = smem;                                              // [BATCH][K]
-    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * a.K);   // 68 floats
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = a.K, N = a.N;
+    int8_t* sx = smem;                                                   // [BATCH][K] permuted INT8 activations
+    int8_t* snx = smem + size_t(BATCH) * K;                              // XSEL: their negation
+    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * K * (XSEL ? 2 : 1));   // 68 floats + BATCH scales
+    float* sxs = red + 68;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: row bases stay in scalar registers
 
     // MoE: one slot per blockIdx.y, its own expert and (xstride = 1) its own input row
     const int slot = blockIdx.y;
@@ -118,94 +141,135 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         expert = (a.shared_expert >= 0 && slot == a.n_eidx) ? a.shared_expert : a.eidx[slot];
         xrow0 = slot * a.xstride;
     }
-    float xs[BATCH];
-#pragma unroll
-    for (int b = 0; b < BATCH; ++b) xs[b] = stage_row<NT>(a, xrow0 + b, sx + size_t(b) * K, red);
-    __syncthreads();
-
-    const int n0 = (blockIdx.x * (NT / 64) + wave) * R;
-    if (n0 >= N) return;
-    const size_t erow = size_t(expert) * N;
-    const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + (erow + n0) * (K / 2);
-    const uint8_t* brow = a.bcodes + (erow + n0) * a.bc_row_bytes;
-
-    int acc[R][BATCH];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int b = 0; b < BATCH; ++b) acc[r][b] = 0;
-
-    const int nchunk = K / 32;   // 16-byte code groups per row
-    for (int c = lane; c < nchunk; c += 64) {
-        u32x4 w[R];
-        uint32_t bc[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            w[r] = *reinterpret_cast<const u32x4*>(crow + size_t(r) * (K / 2) + 16 * c);
-            if (DEFAULT_FMT) bc[r] = (uint32_t(brow[r * a.bc_row_bytes + (c >> 2)]) >> (2 * (c & 3))) & 3u;
-        }
-        u32x4 xv[BATCH][2];
-#pragma unroll
-        for (int b = 0; b < BATCH; ++b) {
-            xv[b][0] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32 * c);
-            xv[b][1] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32 * c + 16);
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int part[BATCH];
-#pragma unroll
-            for (int b = 0; b < BATCH; ++b) part[b] = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint32_t e, o;
-                if (DEFAULT_FMT) {
-                    const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, 0u);   // folds to constants
-                    decode_word_split(w[r][j], t, e, o);
-                } else {
-                    const uint32_t blk = uint32_t(32 * c + 8 * j) >> a.fmt.block_log2;
-                    const uint32_t code = block_code(brow + r * a.bc_row_bytes, blk, a.fmt.bc_bits);
-                    const BlockLut t = scaled_lut_mul(a.fmt.lut_lo, a.fmt.lut_hi, mult_of(a.fmt, code));
-                    decode_word_split(w[r][j], t, e, o);
-                }
-#pragma unroll
-                for (int b = 0; b < BATCH; ++b) {
-                    part[b] = __builtin_amdgcn_sdot4(int(e), int(xv[b][j >> 1][2 * (j & 1)]), part[b], false);
-                    part[b] = __builtin_amdgcn_sdot4(int(o), int(xv[b][j >> 1][2 * (j & 1) + 1]), part[b], false);
-                }
-            }
-#pragma unroll
-            for (int b = 0; b < BATCH; ++b) acc[r][b] += DEFAULT_FMT ? (part[b] << bc[r]) : part[b];
-        }
-    }
-
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int b = 0; b < BATCH; ++b) acc[r][b] = wave_sum_i32(acc[r][b]);
-    if (lane != 0) return;
-
-    const float* ws = a.wscale + erow + n0;
-    const int orow0 = a.eidx ? slot : 0;
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-        float y[R];
+        const float s = stage_row<NT>(a, xrow0 + b, sx + size_t(b) * K, red);
+        if (tid == 0) sxs[b] = s;
+    }
+    __syncthreads();
+    if (XSEL) {
+        for (int c = tid; c < K / 4; c += NT)
+            reinterpret_cast<uint32_t*>(snx)[c] = neg_i8x4(reinterpret_cast<const uint32_t*>(sx)[c]);
+        __syncthreads();
+    }
+
+    // constants kept in vector registers so that (x & k) | k' is one v_and_or_b32
+    uint32_t k_sign = 0x04040404u, k_ident = 0x03020100u;
+    asm volatile("" : "+v"(k_sign), "+v"(k_ident));
+    const size_t erow = size_t(expert) * N;
+    const int orow0 = a.eidx ? slot : 0;
+    const int nchunk = K / 32;   // 16-byte code groups per row
+    const int groups = N / R;
+    // waves walk the row groups with a grid stride, so the staged activations serve many rows
+    for (int g = blockIdx.x * (NT / 64) + wave; g < groups; g += gridDim.x * (NT / 64)) {
+        const int n0 = g * R;
+        const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + (erow + n0) * (K / 2);   // wave-uniform
+        const uint8_t* brow = a.bcodes + (erow + n0) * a.bc_row_bytes;
+        int acc[NV];
 #pragma unroll
-        for (int r = 0; r < R; ++r) y[r] = __fmul_rn(__fmul_rn(float(acc[r][b]), xs[b]), ws[r]);
-        if (a.epi == SCMX_EPI_SCALE) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) a.out[size_t(orow0 + b) * N + n0 + r] = f32_to_bf16(y[r]);
-        } else if (a.epi == SCMX_EPI_RES) {
+        for (int i = 0; i < NV; ++i) acc[i] = 0;
+
+        for (uint32_t c = lane; c < uint32_t(nchunk); c += 64) {
+            u32x4 w[R];
+            uint32_t bc[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const float rv = bf16_to_f32(a.res[size_t(orow0 + b) * N + n0 + r]);
-                a.out[size_t(orow0 + b) * N + n0 + r] = f32_to_bf16(__fadd_rn(rv, round_bf16(y[r])));
+                w[r] = *reinterpret_cast<const u32x4*>(crow + size_t(r) * (K / 2) + 16u * c);
+                if (DEFAULT_FMT) bc[r] = (brow + size_t(r) * a.bc_row_bytes)[c >> 2];
             }
-        } else if (R % 4 == 0) {   // SwiGLU of (g, g, u, u)
+            u32x4 xv[BATCH][2], nxv[2];
 #pragma unroll
-            for (int r = 0; r < R; r += 4) {
-                uint16_t* o = a.out + size_t(orow0 + b) * (N / 2) + (n0 + r) / 2;
-                o[0] = swiglu_bf16(round_bf16(y[r]), round_bf16(y[(r + 2) % R]));
-                o[1] = swiglu_bf16(round_bf16(y[(r + 1) % R]), round_bf16(y[(r + 3) % R]));
+            for (int b = 0; b < BATCH; ++b) {
+                xv[b][0] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32u * c);
+                xv[b][1] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32u * c + 16);
+            }
+            if (XSEL) {
+                nxv[0] = *reinterpret_cast<const u32x4*>(snx + 32u * c);
+                nxv[1] = *reinterpret_cast<const u32x4*>(snx + 32u * c + 16);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                int part[BATCH];
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b) part[b] = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t wj = w[r][j];
+                    if (XSEL) {
+                        // magnitudes from the lookup; signs folded into a per-byte choice between x and -x:
+                        // selector byte i = i + 4 * sign picks byte i of x or of -x
+                        const uint32_t t = wj >> 4;
+                        const uint32_t me = perm(0x0C080604u, 0x03020100u, wj & 0x07070707u);
+                        const uint32_t mo = perm(0x0C080604u, 0x03020100u, t & 0x07070707u);
+                        const uint32_t xe = xv[0][j >> 1][2 * (j & 1)], xo = xv[0][j >> 1][2 * (j & 1) + 1];
+                        const uint32_t ne = nxv[j >> 1][2 * (j & 1)], no = nxv[j >> 1][2 * (j & 1) + 1];
+                        const uint32_t se = perm(ne, xe, ((wj >> 1) & k_sign) | k_ident);   // v_and_or_b32
+                        const uint32_t so = perm(no, xo, ((wj >> 5) & k_sign) | k_ident);
+                        part[0] = __builtin_amdgcn_sdot4(int(me), int(se), part[0], false);
+                        part[0] = __builtin_amdgcn_sdot4(int(mo), int(so), part[0], false);
+                        continue;
+                    }
+                    uint32_t e, o;
+                    if (DEFAULT_FMT) {
+                        const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, 0u);   // folds to constants
+                        decode_word_split(wj, t, e, o);
+                    } else {
+                        const uint32_t blk = uint32_t(32 * c + 8 * j) >> a.fmt.block_log2;
+                        const uint32_t code = block_code(brow + r * a.bc_row_bytes, blk, a.fmt.bc_bits);
+                        const BlockLut t = scaled_lut_mul(a.fmt.lut_lo, a.fmt.lut_hi, mult_of(a.fmt, code));
+                        decode_word_split(wj, t, e, o);
+                    }
+#pragma unroll
+                    for (int b = 0; b < BATCH; ++b) {
+                        part[b] = __builtin_amdgcn_sdot4(int(e), int(xv[b][j >> 1][2 * (j & 1)]), part[b], false);
+                        part[b] = __builtin_amdgcn_sdot4(int(o), int(xv[b][j >> 1][2 * (j & 1) + 1]), part[b], false);
+                    }
+                }
+                const uint32_t sh = DEFAULT_FMT ? (bc[r] >> (2 * (c & 3))) & 3u : 0u;
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b) acc[r * BATCH + b] += part[b] << sh;
+            }
+        }
+
+        // totals land in lane 63, which applies the epilogue to the R x BATCH outputs of this row group
+#pragma unroll
+        for (int i = 0; i < NV; ++i) acc[i] = wave_sum_to_lane63(acc[i]);
+        if (lane == 63) {
+            float wsr[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) wsr[r] = a.wscale[erow + n0 + r];
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) {
+                const float xsb = sxs[b];
+                const size_t orow = size_t(orow0 + b);
+                float y[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) y[r] = __fmul_rn(__fmul_rn(float(acc[r * BATCH + b]), xsb), wsr[r]);
+                if (a.epi == SCMX_EPI_SCALE) {
+                    if (R == 8 && (N & 7) == 0) {   // 8 consecutive outputs: one 16-byte store
+                        u32x4 o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            o[r] = uint32_t(f32_to_bf16(y[(2 * r) % R])) | (uint32_t(f32_to_bf16(y[(2 * r + 1) % R])) << 16);
+                        *reinterpret_cast<u32x4*>(a.out + orow * N + n0) = o;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < R; ++r) a.out[orow * N + n0 + r] = f32_to_bf16(y[r]);
+                    }
+                } else if (a.epi == SCMX_EPI_RES) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const float rv = bf16_to_f32(a.res[orow * N + n0 + r]);
+                        a.out[orow * N + n0 + r] = f32_to_bf16(__fadd_rn(rv, round_bf16(y[r])));
+                    }
+                } else if (R % 4 == 0) {   // SwiGLU of rows (g, g, u, u)
+#pragma unroll
+                    for (int r = 0; r < R; r += 4) {
+                        uint16_t* o = a.out + orow * (N / 2) + (n0 + r) / 2;
+                        o[0] = swiglu_bf16(round_bf16(y[r]), round_bf16(y[(r + 2) % R]));
+                        o[1] = swiglu_bf16(round_bf16(y[(r + 1) % R]), round_bf16(y[(r + 3) % R]));
+                    }
+                }
             }
         }
     }
@@ -213,8 +277,13 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 
 template <int BATCH, int R>
 static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
-    const dim3 grid((a.N / R + 3) / 4, slots), block(256);
-    const size_t smem = size_t(BATCH) * a.K + 68 * sizeof(float);
+    // enough workgroups to fill the chip (4 waves each), but no more than ~16 resident waves per CU: waves loop
+    const int groups = a.N / R;
+    const int want = (groups + 3) / 4;
+    const int cap = max(1, 1024 / slots);
+    const dim3 grid(min(want, cap), slots), block(256);
+    const bool xsel = dflt && BATCH == 1;
+    const size_t smem = size_t(BATCH) * a.K * (xsel ? 2 : 1) + (68 + BATCH) * sizeof(float);
     if (dflt)
         gemv_kernel<BATCH, R, true><<<grid, block, smem, s>>>(a);
     else
@@ -223,10 +292,13 @@ static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) 
 
 template <int BATCH>
 static void launch_gemv_rows(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
-    // more rows per wave = more loads in flight per lane; fewer = more workgroups for narrow layers
+    // more rows per wave = more loads in flight per lane; fewer = more waves for narrow layers
     const long rows = long(a.N) * slots;
-    if (a.epi == SCMX_EPI_SWIGLU || (rows >= 32768 && a.N % 4 == 0)) return launch_gemv<BATCH, 4>(a, slots, dflt, s);
-    if (rows >= 8192 && a.N % 2 == 0) return launch_gemv<BATCH, 2>(a, slots, dflt, s);
+    constexpr int RMAX = BATCH == 1 ? 8 : BATCH == 2 ? 4 : BATCH == 4 ? 2 : 1;   // keeps the kernel near 128 VGPRs
+    if (a.epi == SCMX_EPI_SWIGLU) return launch_gemv<BATCH, 4>(a, slots, dflt, s);
+    if (RMAX >= 8 && rows >= 65536 && a.N % 8 == 0) return launch_gemv<BATCH, RMAX >= 8 ? 8 : 1>(a, slots, dflt, s);
+    if (RMAX >= 4 && rows >= 16384 && a.N % 4 == 0) return launch_gemv<BATCH, RMAX >= 4 ? 4 : 1>(a, slots, dflt, s);
+    if (RMAX >= 2 && rows >= 4096 && a.N % 2 == 0) return launch_gemv<BATCH, RMAX >= 2 ? 2 : 1>(a, slots, dflt, s);
     return launch_gemv<BATCH, 1>(a, slots, dflt, s);
 }
 
@@ -270,7 +342,7 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
         set_error("gemv: batch %d not in {1,2,4,8}", batch);
         return SCMX_ERR_ARG;
     }
-    if (size_t(batch) * K + 68 * sizeof(float) > 64 * 1024) {
+    if (size_t(batch) * K * (batch == 1 ? 2 : 1) + 80 * sizeof(float) > 64 * 1024) {
         set_error("gemv: batch * K = %zu bytes of activations exceed the 64 KiB staged per workgroup", size_t(batch) * K);
         return SCMX_ERR_ARG;
     }
