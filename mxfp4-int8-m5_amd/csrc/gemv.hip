@@ -76,15 +76,29 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
         inv = red[64];
         __syncthreads();
     }
-    auto value = [&](int k) -> float {
-        const float xv = bf16_to_f32(xr[k]);
-        if (a.pro == 2) return round_bf16(__fmul_rn(bf16_to_f32(a.nw[k]), round_bf16(__fmul_rn(xv, inv))));
-        return xv;
+    // eight values per thread and step, from one 16-byte load (and one of the norm weight for pro 2)
+    auto values = [&](int c, float (&v)[8]) {
+        const u32x4 p = *reinterpret_cast<const u32x4*>(xr + 8 * c);
+        u32x4 q = u32x4{0u, 0u, 0u, 0u};
+        if (a.pro == 2) q = *reinterpret_cast<const u32x4*>(a.nw + 8 * c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float xv = __uint_as_float(i & 1 ? (p[i >> 1] & 0xFFFF0000u) : (p[i >> 1] << 16));
+            if (a.pro == 2) {
+                const float wv = __uint_as_float(i & 1 ? (q[i >> 1] & 0xFFFF0000u) : (q[i >> 1] << 16));
+                v[i] = round_bf16(__fmul_rn(wv, round_bf16(__fmul_rn(xv, inv))));
+            } else {
+                v[i] = xv;
+            }
+        }
     };
     float amax = 0.0f;
-    for (int c = tid; c < K / 8; c += NT)
+    for (int c = tid; c < K / 8; c += NT) {
+        float v[8];
+        values(c, v);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(value(8 * c + i)));
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    }
     amax = wave_max(amax);
     if (lane == 0) red[wave] = amax;
     __syncthreads();
@@ -93,9 +107,11 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
     const float s = __fdiv_rn(amax, 127.0f);
     const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
     for (int c = tid; c < K / 8; c += NT) {
+        float v[8];
+        values(c, v);
         int q[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = quant_code(value(8 * c + i), qi);
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], qi);
         store_perm8(sx + 8 * c, q);
     }
     __syncthreads();   // `red` is reused by the next row
@@ -114,6 +130,46 @@ __device__ __forceinline__ int wave_sum_to_lane63(int v) {
     return v;
 }
 
+// Value of `v` in lane (lane ^ OFF): DPP moves where the pattern exists, the LDS crossbar otherwise.
+template <int OFF>
+__device__ __forceinline__ int xor_lane(int v) {
+    if (OFF == 1) return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);    // quad_perm [1,0,3,2]
+    if (OFF == 2) return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);    // quad_perm [2,3,0,1]
+    if (OFF == 4) return __builtin_amdgcn_ds_swizzle(v, 0x101F);                      // bit mode: xor 4
+    if (OFF == 8) return __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, false);   // row_ror:8
+    if (OFF == 16) return __builtin_amdgcn_ds_swizzle(v, 0x401F);                     // bit mode: xor 16
+    return __shfl_xor(v, 32, WAVE);
+}
+
+// Wave totals of NV per-lane values in 6 exchange steps (offsets 1, 2, 4, 8, 16, 32).  While more than one value is
+// left, a step halves the set: lanes whose bit is clear keep the lower half and receive the partner's partials of
+// it, the others the upper half; the remaining steps are plain sums.  Lane L ends with the total of value index
+// bitreverse(L mod NV) over log2(NV) bits; every lane with the same L mod NV holds the same total.
+template <int NV, int OFF = 1>
+__device__ __forceinline__ int select_reduce(int (&v)[NV], int lane) {
+    if constexpr (NV > 1) {
+        const bool up = (lane & OFF) != 0;
+        int h[NV / 2];
+#pragma unroll
+        for (int i = 0; i < NV / 2; ++i) {
+            const int keep = up ? v[i + NV / 2] : v[i];
+            const int send = up ? v[i] : v[i + NV / 2];
+            h[i] = keep + xor_lane<OFF>(send);
+        }
+        if constexpr (OFF < 32) return select_reduce<NV / 2, OFF * 2>(h, lane);
+        else return h[0];
+    } else {
+        int t = v[0];
+        if constexpr (OFF <= 1) t += xor_lane<1>(t);
+        if constexpr (OFF <= 2) t += xor_lane<2>(t);
+        if constexpr (OFF <= 4) t += xor_lane<4>(t);
+        if constexpr (OFF <= 8) t += xor_lane<8>(t);
+        if constexpr (OFF <= 16) t += xor_lane<16>(t);
+        if constexpr (OFF <= 32) t += xor_lane<32>(t);
+        return t;
+    }
+}
+
 // Per-byte negation of INT8 bytes in -127..127.
 __device__ __forceinline__ uint32_t neg_i8x4(uint32_t x) {
     const uint32_t n = ~x;
@@ -128,8 +184,9 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int K = a.K, N = a.N;
     int8_t* sx = smem;                                                   // [BATCH][K] permuted INT8 activations
-    int8_t* snx = smem + size_t(BATCH) * K;                              // XSEL: their negation
-    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * K * (XSEL ? 2 : 1));   // 68 floats + BATCH scales
+    const int Kp = (K + 2047) & ~2047;                                    // row pitch: whole 64-chunk slices, zero padded
+    int8_t* snx = smem + size_t(BATCH) * Kp;                             // XSEL: their negation
+    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * Kp * (XSEL ? 2 : 1));   // 68 floats + BATCH scales
     float* sxs = red + 68;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: row bases stay in scalar registers
@@ -143,12 +200,13 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     }
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-        const float s = stage_row<NT>(a, xrow0 + b, sx + size_t(b) * K, red);
+        const float s = stage_row<NT>(a, xrow0 + b, sx + size_t(b) * Kp, red);
+        for (int c = K / 4 + tid; c < Kp / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
         if (tid == 0) sxs[b] = s;
     }
     __syncthreads();
     if (XSEL) {
-        for (int c = tid; c < K / 4; c += NT)
+        for (int c = tid; c < Kp / 4; c += NT)
             reinterpret_cast<uint32_t*>(snx)[c] = neg_i8x4(reinterpret_cast<const uint32_t*>(sx)[c]);
         __syncthreads();
     }
@@ -160,28 +218,43 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     const int orow0 = a.eidx ? slot : 0;
     const int nchunk = K / 32;   // 16-byte code groups per row
     const int groups = N / R;
-    // waves walk the row groups with a grid stride, so the staged activations serve many rows
-    for (int g = blockIdx.x * (NT / 64) + wave; g < groups; g += gridDim.x * (NT / 64)) {
-        const int n0 = g * R;
-        const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + (erow + n0) * (K / 2);   // wave-uniform
-        const uint8_t* brow = a.bcodes + (erow + n0) * a.bc_row_bytes;
-        int acc[NV];
+    // Waves walk the row groups with a grid stride, so the staged activations serve many rows.  The work of a wave is
+    // a sequence of items (row group, 64-chunk slice of K); the weights of the next item are loaded into a second
+    // register set before the current item is decoded, so every wave always has loads in flight.
+    struct Item {
+        u32x4 w[R];
+        uint32_t bc[R];
+    };
+    const int g_stride = gridDim.x * (NT / 64);
+    const int CI = (nchunk + 63) / 64;                 // items per row group
+    // Buffer loads: the row group's base sits in a scalar resource descriptor, the row offset in a scalar operand and
+    // the lane's chunk offset in one vector register, so a load costs no vector address arithmetic; reads past the
+    // group's last row return zero.
+    auto load_item = [&](Item& it, int g, uint32_t c) {
+        const uint32_t cc = min(c, uint32_t(nchunk - 1));
+        const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + (erow + size_t(g) * R) * (K / 2);   // uniform
+        const uint8_t* brow = a.bcodes + (erow + size_t(g) * R) * a.bc_row_bytes;
+        const __amdgpu_buffer_rsrc_t rc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(crow), 0, R * (K / 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rb =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(brow), 0, R * a.bc_row_bytes, 0x00020000);
 #pragma unroll
-        for (int i = 0; i < NV; ++i) acc[i] = 0;
-
-        for (uint32_t c = lane; c < uint32_t(nchunk); c += 64) {
-            u32x4 w[R];
-            uint32_t bc[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                w[r] = *reinterpret_cast<const u32x4*>(crow + size_t(r) * (K / 2) + 16u * c);
-                if (DEFAULT_FMT) bc[r] = (brow + size_t(r) * a.bc_row_bytes)[c >> 2];
-            }
+        for (int r = 0; r < R; ++r) {
+            it.w[r] = __builtin_amdgcn_raw_buffer_load_b128(rc, int(16u * cc), r * (K / 2), 0);
+            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> 2), r * a.bc_row_bytes, 0);
+        }
+    };
+    auto compute_item = [&](const Item& it, int g, uint32_t c_in, int (&acc)[NV]) {
+        const uint32_t c = c_in;   // lanes past the row end read activations from the zero padding in LDS
+        const u32x4(&w)[R] = it.w;
+        const uint32_t(&bc)[R] = it.bc;
+        const uint8_t* brow = a.bcodes + (erow + size_t(g) * R) * a.bc_row_bytes;
+        (void)brow;
             u32x4 xv[BATCH][2], nxv[2];
 #pragma unroll
             for (int b = 0; b < BATCH; ++b) {
-                xv[b][0] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32u * c);
-                xv[b][1] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * K + 32u * c + 16);
+                xv[b][0] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * Kp + 32u * c);
+                xv[b][1] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * Kp + 32u * c + 16);
             }
             if (XSEL) {
                 nxv[0] = *reinterpret_cast<const u32x4*>(snx + 32u * c);
@@ -229,9 +302,27 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 #pragma unroll
                 for (int b = 0; b < BATCH; ++b) acc[r * BATCH + b] += part[b] << sh;
             }
-        }
 
-        // totals land in lane 63, which applies the epilogue to the R x BATCH outputs of this row group
+    };
+    auto finish = [&](int g, int (&acc)[NV]) {
+        const int n0 = g * R;
+        if (a.epi != SCMX_EPI_SWIGLU) {
+            // one output per lane: lane L < NV ends with the total of value index bitreverse(L), r * BATCH + b
+            const int tot = select_reduce<NV>(acc, lane);
+            if (lane < NV) {
+                constexpr int LOG = NV == 1 ? 0 : NV == 2 ? 1 : NV == 4 ? 2 : NV == 8 ? 3 : NV == 16 ? 4 : NV == 32 ? 5 : 6;
+                const int idx = LOG == 0 ? 0 : int(__builtin_bitreverse32(uint32_t(lane)) >> (32 - (LOG == 0 ? 1 : LOG)));
+                const int r = idx / BATCH, b = idx % BATCH;
+                const float y = __fmul_rn(__fmul_rn(float(tot), sxs[b]), a.wscale[erow + n0 + r]);
+                const size_t o = size_t(orow0 + b) * N + n0 + r;
+                if (a.epi == SCMX_EPI_SCALE)
+                    a.out[o] = f32_to_bf16(y);
+                else
+                    a.out[o] = f32_to_bf16(__fadd_rn(bf16_to_f32(a.res[o]), round_bf16(y)));
+            }
+            return;
+        }
+        // SwiGLU needs four rows in one lane: totals land in lane 63, which applies the epilogue
 #pragma unroll
         for (int i = 0; i < NV; ++i) acc[i] = wave_sum_to_lane63(acc[i]);
         if (lane == 63) {
@@ -272,6 +363,38 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
                 }
             }
         }
+    };
+
+    int g = blockIdx.x * (NT / 64) + wave;
+    if (g >= groups) return;
+    int ci = 0;
+    int acc[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = 0;
+    Item ia, ib;
+    load_item(ia, g, lane);
+    // one step: prefetch the next item into `nxt`, decode `cur`; returns false after the wave's last item
+    auto step = [&](const Item& cur, Item& nxt) {
+        int ng = g, nci = ci + 1;
+        if (nci == CI) {
+            nci = 0;
+            ng = g + g_stride;
+        }
+        const bool more = ng < groups;
+        load_item(nxt, more ? ng : g, lane + 64u * (more ? nci : ci));
+        compute_item(cur, g, lane + 64u * ci, acc);
+        if (ci == CI - 1) {
+            finish(g, acc);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) acc[i] = 0;
+        }
+        g = ng;
+        ci = nci;
+        return more;
+    };
+    while (true) {
+        if (!step(ia, ib)) break;
+        if (!step(ib, ia)) break;
     }
 }
 
@@ -283,7 +406,7 @@ static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) 
     const int cap = max(1, 1024 / slots);
     const dim3 grid(min(want, cap), slots), block(256);
     const bool xsel = dflt && BATCH == 1;
-    const size_t smem = size_t(BATCH) * a.K * (xsel ? 2 : 1) + (68 + BATCH) * sizeof(float);
+    const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (xsel ? 2 : 1) + (68 + BATCH) * sizeof(float);
     if (dflt)
         gemv_kernel<BATCH, R, true><<<grid, block, smem, s>>>(a);
     else
@@ -294,9 +417,8 @@ template <int BATCH>
 static void launch_gemv_rows(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
     // more rows per wave = more loads in flight per lane; fewer = more waves for narrow layers
     const long rows = long(a.N) * slots;
-    constexpr int RMAX = BATCH == 1 ? 8 : BATCH == 2 ? 4 : BATCH == 4 ? 2 : 1;   // keeps the kernel near 128 VGPRs
+    constexpr int RMAX = BATCH == 1 ? 4 : BATCH == 2 ? 4 : BATCH == 4 ? 2 : 1;   // keeps several waves per SIMD resident
     if (a.epi == SCMX_EPI_SWIGLU) return launch_gemv<BATCH, 4>(a, slots, dflt, s);
-    if (RMAX >= 8 && rows >= 65536 && a.N % 8 == 0) return launch_gemv<BATCH, RMAX >= 8 ? 8 : 1>(a, slots, dflt, s);
     if (RMAX >= 4 && rows >= 16384 && a.N % 4 == 0) return launch_gemv<BATCH, RMAX >= 4 ? 4 : 1>(a, slots, dflt, s);
     if (RMAX >= 2 && rows >= 4096 && a.N % 2 == 0) return launch_gemv<BATCH, RMAX >= 2 ? 2 : 1>(a, slots, dflt, s);
     return launch_gemv<BATCH, 1>(a, slots, dflt, s);
@@ -325,8 +447,8 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
         set_error("gemv: need K %% 128 == 0, whole block-code bytes per row, N %% 4 == 0 for SwiGLU (N=%d K=%d)", N, K);
         return SCMX_ERR_ARG;
     }
-    if (uintptr_t(codes) % 16 || uintptr_t(x) % 8) {
-        set_error("gemv: codes must be 16-byte aligned, x 8-byte aligned");
+    if (uintptr_t(codes) % 16 || uintptr_t(x) % 16 || (pro == 2 && uintptr_t(nw) % 16)) {
+        set_error("gemv: codes, x and nw must be 16-byte aligned");
         return SCMX_ERR_ARG;
     }
     int slots = 1;
@@ -342,7 +464,7 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
         set_error("gemv: batch %d not in {1,2,4,8}", batch);
         return SCMX_ERR_ARG;
     }
-    if (size_t(batch) * K * (batch == 1 ? 2 : 1) + 80 * sizeof(float) > 64 * 1024) {
+    if (size_t(batch) * ((K + 2047) & ~2047) * (batch == 1 ? 2 : 1) + 80 * sizeof(float) > 64 * 1024) {
         set_error("gemv: batch * K = %zu bytes of activations exceed the 64 KiB staged per workgroup", size_t(batch) * K);
         return SCMX_ERR_ARG;
     }
