@@ -22,6 +22,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0        # MI355X dense INT8 MFMA, published
+# HBM-side bytes per GEMM launch (mean over the four layer launches of one step), from rocprofv3 TCC counters of this
+# workload: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, both factors calibrated on a 256 MiB device copy.  Per layer
+# (fetched + written MiB): qkv 36.4 + 16, o_proj 34.3 + 8, gate_up 108.7 + 48, down 102.4 + 8.
+GEMM_TRAFFIC_BYTES = int((36.4 + 16 + 34.3 + 8 + 108.7 + 48 + 102.4 + 8) * 2 ** 20 / 4)
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E, published
 M_TOKENS = 2048
 LAYERS = [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]
@@ -80,6 +84,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV leg")
+    ap.add_argument("--profile-copy", action="store_true",
+                    help="first run one plain 256 MiB device copy: the known-size kernel that calibrates FETCH_SIZE / "
+                         "WRITE_SIZE when this command runs under rocprofv3 --pmc")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
@@ -100,6 +107,13 @@ def main():
         if arr.dtype == np.uint32:
             arr = arr.view(np.int32)
         return torch.from_numpy(arr).to(dev)
+
+    if a.profile_copy:
+        src = torch.empty(256 * 2 ** 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- prefill: weight sets rotate (> 256 MB in total, beyond the last-level cache) --------------------------
     set_bytes = sum(n * k // 2 + n * k // 128 + 4 * n for _, n, k in LAYERS)
@@ -170,7 +184,7 @@ def main():
         tot_ms += ms
     achieved = tot_ops / tot_ms / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None, "kernel": "scmx::gemm_kernel (mm_w4a8)",
+                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": GEMM_TRAFFIC_BYTES, "kernel": "scmx::gemm_kernel (mm_w4a8)",
                 "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their average launch "
                         "durations, activations pre-quantized", "per_shape": per_shape}
 
