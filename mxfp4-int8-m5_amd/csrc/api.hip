@@ -160,6 +160,51 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
     if (tid == 0) xs[row] = s;
 }
 
+// The same with the row held in registers: one wave per row, lane l owns the 16-byte pieces l, l + 64, ... (CH of
+// them, K = 512 * CH), so the row is read once and the only reduction is inside the wave.  Four rows per workgroup.
+template <int CH>
+__global__ __launch_bounds__(256) void act_quant_wave_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
+                                                             float* __restrict__ xs, int M, int Mp) {
+    constexpr int K = 512 * CH;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= Mp) return;
+    u32x2* qrow = reinterpret_cast<u32x2*>(xq + size_t(row) * K);
+    if (row >= M) {
+#pragma unroll
+        for (int j = 0; j < CH; ++j) qrow[lane + 64 * j] = u32x2{0u, 0u};
+        if (lane == 0) xs[row] = 0.0f;
+        return;
+    }
+    const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
+    u32x4 v[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) v[j] = xrow[lane + 64 * j];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            amax = fmaxf(amax, fabsf(__uint_as_float(v[j][e] << 16)));
+            amax = fmaxf(amax, fabsf(__uint_as_float(v[j][e] & 0xFFFF0000u)));
+        }
+    amax = wave_max(amax);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+        uint32_t o[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int q0 = quant_code(__uint_as_float(v[j][e] << 16), qi);
+            const int q1 = quant_code(__uint_as_float(v[j][e] & 0xFFFF0000u), qi);
+            o[e >> 1] |= (uint32_t(q0) & 0xFFu) << (16 * (e & 1));
+            o[e >> 1] |= (uint32_t(q1) & 0xFFu) << (16 * (e & 1) + 8);
+        }
+        qrow[lane + 64 * j] = u32x2{o[0], o[1]};
+    }
+    if (lane == 0) xs[row] = s;
+}
+
 // ---- standard MXFP4 -> block codes + row scale: one wave per row -----------------------------------------------
 __global__ __launch_bounds__(256) void mxfp4_to_sc_kernel(const uint8_t* __restrict__ e8m0,
                                                           uint8_t* __restrict__ bcodes, float* __restrict__ wscale,
@@ -242,7 +287,19 @@ int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int 
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
-    act_quant_kernel<<<dim3(Mp), dim3(256), 0, (hipStream_t)stream>>>(x, xq, xs, M, K);
+    const dim3 wgrid((Mp + 3) / 4), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    switch (K % 512 ? 0 : K / 512) {   // rows of up to 8192 elements stay in registers
+        case 1: act_quant_wave_kernel<1><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 2: act_quant_wave_kernel<2><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 3: act_quant_wave_kernel<3><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 4: act_quant_wave_kernel<4><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 6: act_quant_wave_kernel<6><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 8: act_quant_wave_kernel<8><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 12: act_quant_wave_kernel<12><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 16: act_quant_wave_kernel<16><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        default: act_quant_kernel<<<dim3(Mp), block, 0, st>>>(x, xq, xs, M, K); break;
+    }
     return check_launch("act_quant");
 }
 

@@ -6,8 +6,8 @@
 // are written to LDS, so the INT8 form of the weights exists only there.  Waves then read 16-byte operand
 // fragments and issue v_mfma_i32_32x32x32_i8 with the weights as the row operand: each lane ends up with groups
 // of 4 consecutive output columns n of one token row m, which is the unit every epilogue works on.
-// LDS is double buffered: global loads for step i+1 are issued before the MFMAs of step i, decoded and stored
-// after them, with one barrier per step.
+// LDS holds three stages of the K loop; global loads run four steps ahead in two register sets, and the decode and
+// LDS writes of step i+2 are issued between the MFMAs of step i, with one barrier per step.
 #include <type_traits>
 
 #include "scmx_common.h"
@@ -35,10 +35,10 @@ struct GemmArgs {
 
 enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2 };
 
-constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
-
-template <int BM, int BN, int BK, int WGM, int WGN, int BMODE>
-__global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
+// FD = number of fragment register buffers: fragments are fetched FD - 1 k slices ahead of their MFMAs.
+template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2>
+__global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs a) {
+    constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
     constexpr int NT = WGM * WGN * 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int MI = WTM / 32, NI = WTN / 32;
@@ -47,13 +47,19 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
     constexpr int RPB = 256 / BK;            // rows per 256 bytes, i.e. per sweep of the 64 LDS banks
     constexpr int A_CHUNKS = BM * CPR;       // 16-byte pieces of the activation tile
     constexpr int A_PER = (A_CHUNKS + NT - 1) / NT;
-    constexpr int B_CHUNKS = BMODE == B_INT8 ? BN * CPR : BN * BK / 32;   // 16 bytes of INT8 or of codes
+    // packed weights are staged in runs of 8 * WPC weights (WPC code words) per thread: 32 when that keeps every
+    // thread busy, else 16
+    constexpr int WPC = BN * BK / 32 >= NT ? 4 : 2;
+    constexpr int B_CHUNKS = BMODE == B_INT8 ? BN * CPR : BN * BK / (8 * WPC);
     constexpr int B_PER = (B_CHUNKS + NT - 1) / NT;
     constexpr int STAGE = (BM + BN) * BK;    // bytes per stage: BM activation rows then BN weight rows
 
     // Rows are BK bytes with no padding; the 16-byte chunk c of row r sits at chunk c ^ ((r / RPB) % CPR), which
     // spreads the 16 rows a b128 fragment read touches per pass over all 64 banks.
     __shared__ __attribute__((aligned(16))) int8_t smem[NSTAGE * STAGE];
+    // scales of the tile's rows and columns, fetched before the K loop so that the epilogue does not start with a
+    // round trip to memory
+    __shared__ __attribute__((aligned(16))) float s_xs[BM], s_ws[BN];
     auto swz = [](int row, int chunk) { return row * BK + ((chunk ^ ((row / RPB) & (CPR - 1))) << 4); };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -85,76 +91,106 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
         row_end = a.M;
     }
     const int K = a.K;
+    if (a.xscale) {   // published by the barrier that opens the K loop
+        for (int r = tid; r < BM; r += NT) {
+            const int m = m0 + r;
+            s_xs[r] = m < row_end ? a.xscale[a.gather ? a.gather[m] : m] : 0.0f;
+        }
+        for (int c = tid; c < BN; c += NT) s_ws[c] = n0 + c < a.N ? a.wscale[size_t(expert) * a.N + n0 + c] : 0.0f;
+    }
 
     // ---- per-thread staging assignments (fixed over the K loop) ------------------------------------------------
-    const int8_t* a_src[A_PER];
-    int a_dst[A_PER];
+    // Global operands are read with buffer loads: a per-thread byte offset fixed for the whole K loop plus a scalar
+    // offset that advances with k, so the loop spends no vector instructions on addresses.
+    const auto rsrc = [](const void* p, size_t bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, int(bytes), 0x00020000);
+    };
+    const size_t erow = size_t(expert) * a.N;   // first weight row of this expert
+    const __amdgpu_buffer_rsrc_t ra = rsrc(a.xq, 0xFFFFFFFFu);
+    const __amdgpu_buffer_rsrc_t rb = BMODE == B_INT8 ? rsrc(a.wq + erow * K, size_t(a.N) * K)
+                                                      : rsrc(reinterpret_cast<const uint8_t*>(a.codes) + erow * (K / 2), size_t(a.N) * (K / 2));
+    const __amdgpu_buffer_rsrc_t rbc = rsrc(a.bcodes + erow * a.bc_row_bytes, size_t(a.N) * a.bc_row_bytes);
+    int a_src[A_PER], a_dst[A_PER];
 #pragma unroll
     for (int j = 0; j < A_PER; ++j) {
         const int c = tid + j * NT;
         const int row = c / CPR, kc = c % CPR;
         int gr = min(m0 + row, a.M - 1);
         if (a.gather) gr = a.gather[gr];
-        a_src[j] = a.xq + size_t(gr) * K + kc * 16;
+        a_src[j] = int(uint32_t(gr) * uint32_t(K) + kc * 16);
         a_dst[j] = swz(row, kc);
     }
-    const uint8_t* b_src[B_PER];
-    const uint8_t* b_bc[B_PER];
-    int b_dst[B_PER], b_dst2[B_PER], b_k[B_PER];
+    int b_src[B_PER], b_bc[B_PER], b_dst[B_PER], b_dst2[B_PER], b_k[B_PER];
 #pragma unroll
     for (int j = 0; j < B_PER; ++j) {
         const int c = tid + j * NT;
         if (BMODE == B_INT8) {
             const int row = c / CPR, kc = c % CPR;
             const int gn = min(n0 + row, a.N - 1);
-            b_src[j] = reinterpret_cast<const uint8_t*>(a.wq) + (size_t(expert) * a.N + gn) * K + kc * 16;
+            b_src[j] = gn * K + kc * 16;
             b_dst[j] = BM * BK + swz(row, kc);
             b_dst2[j] = 0;
-            b_bc[j] = nullptr;
+            b_bc[j] = 0;
             b_k[j] = 0;
         } else {
-            const int row = c / (BK / 32), kb = c % (BK / 32);
+            constexpr int RUNS = BK / (8 * WPC);   // runs per tile row
+            const int row = c / RUNS, kb = c % RUNS;
             const int gn = min(n0 + row, a.N - 1);
-            b_src[j] = reinterpret_cast<const uint8_t*>(a.codes) + (size_t(expert) * a.N + gn) * (K / 2) + kb * 16;
-            b_bc[j] = a.bcodes + (size_t(expert) * a.N + gn) * a.bc_row_bytes;
-            b_dst[j] = BM * BK + swz(row, 2 * kb);
-            b_dst2[j] = BM * BK + swz(row, 2 * kb + 1);
-            b_k[j] = kb * 32;
+            b_src[j] = gn * (K / 2) + kb * 4 * WPC;
+            b_bc[j] = gn * a.bc_row_bytes;
+            b_dst[j] = BM * BK + swz(row, kb * WPC / 2);
+            b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
+            b_k[j] = kb * 8 * WPC;
         }
     }
 
     // Two register sets hold the global loads of two K steps in flight.
     struct Staged {
         u32x4 a[A_PER], b[B_PER];
-        uint32_t bc[B_PER];
+        uint8_t bc[B_PER];   // kept as loaded: widening it here would make the compiler wait for the load at once
     };
     Staged r0, r1;
 
     // Loads past the last K step re-read the last step (never consumed): every iteration issues the same loads, so
     // the wait before a register set is used covers exactly that set and not the younger one.
-    auto load_global = [&](Staged& r, int k0) {
-        k0 = min(k0, K - BK);
+    // The loads of one K step are issued in NKK slices (activation chunks j with j % NKK == q in slice q, the
+    // weight words in the last one) so that the K loop can spread them between its MFMAs.
+    constexpr int NKK = BK / 32;
+    auto load_slice = [&](Staged& r, int k0, int q) {
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
-            if (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS)
-                r.a[j] = *reinterpret_cast<const u32x4*>(a_src[j] + k0);
+            if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS))
+                r.a[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_src[j], k0, 0);
+        if (q != NKK - 1) return;
 #pragma unroll
         for (int j = 0; j < B_PER; ++j)
             if (B_CHUNKS % NT == 0 || tid + j * NT < B_CHUNKS) {
                 if (BMODE == B_INT8) {
-                    r.b[j] = *reinterpret_cast<const u32x4*>(b_src[j] + k0);
+                    r.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_src[j], k0, 0);
                 } else {
-                    r.b[j] = *reinterpret_cast<const u32x4*>(b_src[j] + (k0 >> 1));
+                    if (WPC == 4) {
+                        r.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_src[j], k0 >> 1, 0);
+                    } else {
+                        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rb, b_src[j], k0 >> 1, 0);
+                        r.b[j][0] = v[0];
+                        r.b[j][1] = v[1];
+                    }
                     if (BMODE == B_PACKED_DEFAULT)   // 32-blocks, 2-bit codes, 4 blocks per byte: keep the raw byte
-                        r.bc[j] = b_bc[j][uint32_t(k0 + b_k[j]) >> 7];
+                        r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 7, 0);
                 }
             }
+    };
+    // Loads past the last K step re-read the last step (never consumed): every iteration issues the same loads, so
+    // the wait before a register set is used covers exactly that set and not the younger one.
+    auto load_global = [&](Staged& r, int k0) {
+        k0 = min(k0, K - BK);
+#pragma unroll
+        for (int q = 0; q < NKK; ++q) load_slice(r, k0, q);
     };
 
     // Staging work of one K step, cut into NKK slices so that it can be issued in the shadow of the MFMAs of the
     // step being multiplied: slice q writes the activation chunks j with j % NKK == q and decodes the weight code
     // words w with w * NKK / 4 == q; the last slice writes the decoded weights.
-    constexpr int NKK = BK / 32;
     auto stage_slice = [&](const Staged& r, int8_t* st, int k0, int q, uint32_t (&o)[B_PER][8]) {
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
@@ -167,22 +203,22 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
                     if (q == 0) *reinterpret_cast<u32x4*>(st + b_dst[j]) = r.b[j];
                 } else {
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        if (w * NKK / 4 != q) continue;
+                    for (int w = 0; w < WPC; ++w) {
+                        if (w * NKK / WPC != q) continue;
                         if (BMODE == B_PACKED_DEFAULT) {
                             const uint32_t blk = uint32_t(k0 + b_k[j]) >> 5;
-                            const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, (r.bc[j] >> (2 * (blk & 3))) & 3u);
+                            const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, (uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u);
                             decode_word(r.b[j][w], t, o[j][2 * w], o[j][2 * w + 1]);
                         } else {
                             const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> a.fmt.block_log2;
-                            const uint32_t bc = block_code(b_bc[j], blk, a.fmt.bc_bits);
+                            const uint32_t bc = block_code(a.bcodes + erow * a.bc_row_bytes + b_bc[j], blk, a.fmt.bc_bits);
                             const BlockLut t = scaled_lut_mul(a.fmt.lut_lo, a.fmt.lut_hi, mult_of(a.fmt, bc));
                             decode_word(r.b[j][w], t, o[j][2 * w], o[j][2 * w + 1]);
                         }
                     }
-                    if (q == NKK - 1) {
+                    if (q == (WPC - 1) * NKK / WPC) {
                         *reinterpret_cast<u32x4*>(st + b_dst[j]) = u32x4{o[j][0], o[j][1], o[j][2], o[j][3]};
-                        *reinterpret_cast<u32x4*>(st + b_dst2[j]) = u32x4{o[j][4], o[j][5], o[j][6], o[j][7]};
+                        if (WPC == 4) *reinterpret_cast<u32x4*>(st + b_dst2[j]) = u32x4{o[j][4], o[j][5], o[j][6], o[j][7]};
                     }
                 }
             }
@@ -212,59 +248,96 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
     const int a_frag = (wm * WTM + lr) * BK;
     const int b_frag = BM * BK + (wn * WTN + lr) * BK;
 
+    const int KT = K / BK;
     // Pipeline.  Iteration kt: barrier; multiply step kt out of its LDS stage while the register set holding step
     // kt+2 is decoded and written into its stage, one slice per 32-wide k slice of MFMAs; then reissue that set's
-    // global loads for step kt+4.  A stage is rewritten two barriers after its last read and read two barriers after
-    // it was written; global loads have two iterations to land.
-    const int KT = K / BK;
+    // global loads for step kt+4.  A stage is rewritten two barriers after its last read and readable one barrier
+    // after it was written, so the first fragments of step kt+1 are fetched at the end of iteration kt, ahead of the
+    // barrier that opens kt+1.  The stage indices are compile-time constants (the loop is unrolled over the
+    // 3 stages x 2 register sets), which keeps every LDS address an immediate offset from a fixed register.
     load_global(r0, 0);
     load_global(r1, BK);
     store_lds(r0, 0, 0);
     store_lds(r1, 1, BK);
     load_global(r0, 2 * BK);
     load_global(r1, 3 * BK);
-    int rd = 0;   // stage of step kt
-    auto load_frags = [&](const int8_t* src, int kk, v4i (&fa)[MI], v4i (&fb)[NI]) {
+    // Fragments are fetched FD - 1 k slices ahead of the MFMAs that use them, into FD rotating register buffers; the
+    // slices fetched at the end of an iteration belong to the next step's stage.
+    constexpr int AHEAD = FD - 1;
+    static_assert(AHEAD >= 1 && AHEAD <= NKK, "fragment prefetch distance");
+    v4i fa[FD][MI], fb[FD][NI];
+    auto load_frags = [&](const int8_t* src, int kk, v4i (&xa)[MI], v4i (&xb)[NI]) {
 #pragma unroll
-        for (int i = 0; i < MI; ++i) fa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
+        for (int i = 0; i < MI; ++i) xa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
 #pragma unroll
-        for (int j = 0; j < NI; ++j) fb[j] = *reinterpret_cast<const v4i*>(src + b_frag + j * 32 * BK + koff[kk]);
+        for (int j = 0; j < NI; ++j) xb[j] = *reinterpret_cast<const v4i*>(src + b_frag + j * 32 * BK + koff[kk]);
     };
-    auto iteration = [&](Staged& r, int kt) {
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < AHEAD; ++q) load_frags(smem, q, fa[q], fb[q]);
+    auto iteration = [&](auto step_tag, Staged& r, int kt) {
+        constexpr int rd = decltype(step_tag)::value;        // kt % 3: stage of step kt
+        constexpr int wr = (rd + 2) % NSTAGE;                // stage of step kt + 2
+        constexpr int nx = (rd + 1) % NSTAGE;                // stage of step kt + 1
+        constexpr int ph = (NKK * rd) % FD;                  // fragment buffer of slice 0 of this step (FD divides 6 * NKK)
         __syncthreads();
-        const int wr = rd == 0 ? NSTAGE - 1 : rd - 1;   // (kt + 2) % 3
         const int8_t* src = smem + rd * STAGE;
+        const int8_t* nxt = smem + nx * STAGE;
         int8_t* dst = smem + wr * STAGE;
         const int k2 = min((kt + 2) * BK, K - BK);      // past the end: rewrites a stage nobody reads again
+        const int k4 = min((kt + 4) * BK, K - BK);
         uint32_t o[B_PER][8];
-        v4i fa[2][MI], fb[2][NI];
-        load_frags(src, 0, fa[0], fb[0]);
 #pragma unroll
         for (int kk = 0; kk < NKK; ++kk) {
-            if (kk + 1 < NKK) load_frags(src, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+            if (kk + AHEAD < NKK)
+                load_frags(src, kk + AHEAD, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
+            else
+                load_frags(nxt, kk + AHEAD - NKK, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
+            if (FD > 2) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], fa[(ph + kk) % FD][i], acc[i][j], 0, 0, 0);
             stage_slice(r, dst, k2, kk, o);
+            if (FD > 2) __builtin_amdgcn_sched_barrier(0);
         }
-        load_global(r, (kt + 4) * BK);
-        rd = rd == NSTAGE - 1 ? 0 : rd + 1;
+        load_global(r, k4);
     };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    // Whole trips of 6 steps run without an exit inside; the remaining steps are nested so that every copy of the
+    // iteration has exactly one predecessor.  (With merging paths the compiler must assume the fewest outstanding
+    // loads of any path when it places its waits, and ends up waiting for loads issued one step ago.)
     int kt = 0;
-    for (; kt + 1 < KT; kt += 2) {
-        iteration(r0, kt);
-        iteration(r1, kt + 1);
+    for (; kt + 6 <= KT; kt += 6) {
+        iteration(S0{}, r0, kt);
+        iteration(S1{}, r1, kt + 1);
+        iteration(S2{}, r0, kt + 2);
+        iteration(S0{}, r1, kt + 3);
+        iteration(S1{}, r0, kt + 4);
+        iteration(S2{}, r1, kt + 5);
     }
-    if (kt < KT) iteration(r0, kt);
+    if (kt < KT) {
+        iteration(S0{}, r0, kt);
+        if (kt + 1 < KT) {
+            iteration(S1{}, r1, kt + 1);
+            if (kt + 2 < KT) {
+                iteration(S2{}, r0, kt + 2);
+                if (kt + 3 < KT) {
+                    iteration(S0{}, r1, kt + 3);
+                    if (kt + 4 < KT) iteration(S1{}, r0, kt + 4);
+                }
+            }
+        }
+    }
 
     // ---- epilogue ---------------------------------------------------------------------------------------------
     // Lane holds acc[i][j][4g + r] = (m = i*32 + lane%32, n = j*32 + 8g + 4(lane/32) + r) of its wave tile: 4 consecutive
     // columns of one row, the unit every epilogue works on.  Results go through a per-wave LDS tile so that global
     // stores are 16 bytes per lane over whole contiguous row segments.
     const int N = a.N;
-    const float* ws = a.wscale + size_t(expert) * N;
     __syncthreads();   // every wave is done reading the staging buffers
     auto epilogue = [&](auto epi_tag) {
     constexpr int epi = decltype(epi_tag)::value;
@@ -279,22 +352,16 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
     const bool wide = fits && (size_t(on) * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 &&
                       (epi != SCMX_EPI_RES || reinterpret_cast<uintptr_t>(a.res) % 16 == 0);
 
-    // all scale loads of the wave tile are issued together, ahead of the conversions that use them
     float xsv[MI];
     f32x4 wsv[NI][4];
     if (epi != SCMX_EPI_I32) {
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            const int m = wm0 + i * 32 + lr;
-            xsv[i] = m < row_end ? a.xscale[a.gather ? a.gather[m] : m] : 0.0f;
-        }
+        for (int i = 0; i < MI; ++i) xsv[i] = s_xs[wm * WTM + i * 32 + lr];
 #pragma unroll
         for (int j = 0; j < NI; ++j)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = wn0 + j * 32 + 8 * g + 4 * half;
-                wsv[j][g] = n < N ? *reinterpret_cast<const f32x4*>(ws + n) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            }
+            for (int g = 0; g < 4; ++g)
+                wsv[j][g] = *reinterpret_cast<const f32x4*>(&s_ws[wn * WTN + j * 32 + 8 * g + 4 * half]);
     }
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
@@ -397,24 +464,24 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_kernel(const GemmArgs a) {
 
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WGM, int WGN>
+template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2>
 static void launch_tile(const GemmArgs& a, int bmode, int row_tiles, hipStream_t s) {
     const int num_n = (a.N + BN - 1) / BN;
     const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * 64);
     if (bmode == B_INT8)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8><<<grid, block, 0, s>>>(a);
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD><<<grid, block, 0, s>>>(a);
     else if (bmode == B_PACKED_DEFAULT)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT><<<grid, block, 0, s>>>(a);
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD><<<grid, block, 0, s>>>(a);
     else
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC><<<grid, block, 0, s>>>(a);
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD><<<grid, block, 0, s>>>(a);
 }
 
 // Dense: the largest tile that still gives every CU a workgroup.
 static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     const long cus = 256;
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-    if (tiles(256, 128) >= cus) return launch_tile<256, 128, 128, 4, 2>(a, bmode, (a.M + 255) / 256, s);
-    if (tiles(256, 64) >= cus) return launch_tile<256, 64, 128, 4, 2>(a, bmode, (a.M + 255) / 256, s);
+    if (tiles(256, 128) >= cus) return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
+    if (tiles(256, 64) >= cus) return launch_tile<256, 64, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
     if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
     if (tiles(128, 64) >= cus) return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
     return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
@@ -424,6 +491,11 @@ static int check_gemm_common(const char* who, int M, int N, int K, int epi, bool
                              const float* xscale, const float* wscale, const uint16_t* res, const void* out) {
     if (M < 0 || N <= 0 || K <= 0 || K % 128 || N % 4) {
         set_error("%s: need M >= 0, N %% 4 == 0 and K %% 128 == 0 (M=%d N=%d K=%d)", who, M, N, K);
+        return SCMX_ERR_ARG;
+    }
+    if (uint64_t(M) * uint64_t(K) > 0xFFFFFFFFull || uint64_t(N) * uint64_t(K) > 0x7FFFFFFFull) {
+        set_error("%s: operands beyond the 32-bit offsets of the kernel (M*K = %llu, N*K = %llu)", who,
+                  (unsigned long long)(uint64_t(M) * K), (unsigned long long)(uint64_t(N) * K));
         return SCMX_ERR_ARG;
     }
     if (epi < 0 || epi > 3) {
