@@ -84,6 +84,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV leg")
+    ap.add_argument("--no-moe", action="store_true", help="skip the grouped mixture-of-experts leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the M = 512 / 8192 prefill sweep")
     ap.add_argument("--profile-copy", action="store_true",
                     help="first run one plain 256 MiB device copy: the known-size kernel that calibrates FETCH_SIZE / "
                          "WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -188,6 +190,81 @@ def main():
                 "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their average launch "
                         "durations, activations pre-quantized", "per_shape": per_shape}
 
+    # ---- prefill sweep over M (config 1's other token counts): GEMM kernel alone, per shape ---------------------------
+    sweep = {}
+    if not a.no_sweep:
+        for m in (512, 8192):
+            for li, (name, n, k) in enumerate(LAYERS):
+                x = up(acts(rng, m, k)).to(torch.bfloat16)
+                xq = torch.empty((m, k), dtype=torch.int8, device=dev)
+                xs = torch.empty(m, dtype=torch.float32, device=dev)
+                out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+                check(lib.scmx_act_quant(x.data_ptr(), xq.data_ptr(), xs.data_ptr(), m, m, k, sp))
+                argl = []
+                for s in sets:
+                    codes, bc, ws = s[li]
+                    argl.append((C.byref(fmt), xq.data_ptr(), xs.data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(),
+                                 None, out.data_ptr(), 1, m, n, k, sp))
+                for i in range(3):
+                    check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
+                torch.cuda.synchronize()
+                reps_s = 20
+                e0.record(stream)
+                for i in range(reps_s):
+                    check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
+                e1.record(stream)
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / reps_s
+                ops = 2.0 * m * n * k
+                sweep[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
+                                         "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
+                del x, xq, xs, out
+
+    # ---- grouped mixture-of-experts prefill (config 3: 64 experts, top-8, hidden 2048, intermediate 1024, 4096 tokens) ---
+    moe = {}
+    if not a.no_moe:
+        from mxfp4_int8_m5_amd import sc_kernels as SK, sc_moe as SM
+        T, E, TOPK, D, Fi, TM = 4096, 64, 8, 2048, 1024, int(os.environ.get('SCMX_BENCH_TM', '256'))
+        R = T * TOPK
+        logits = rng.standard_normal((T, E)) + rng.standard_normal(E) * 1.5      # biased router: skewed expert loads
+        inds_np = np.argsort(-logits, axis=1)[:, :TOPK]
+        p = np.exp(np.take_along_axis(logits, inds_np, 1))
+        scores = up((p / p.sum(1, keepdims=True)).astype(np.float32)).to(torch.bfloat16)
+        inds = up(inds_np.astype(np.int32))
+        x = up(acts(rng, T, D)).to(torch.bfloat16)
+
+        def experts(n, k):
+            parts = [packed_random(rng, n, k) for _ in range(E)]
+            return (up(np.stack([q[0] for q in parts])), up(np.stack([q[1] for q in parts])),
+                    up(np.stack([q[2] for q in parts])))
+        gu, dn = experts(2 * Fi, D), experts(D, Fi)       # gate|up rows interleaved for the SwiGLU epilogue
+
+        def moe_pass():
+            xq, xs = SK.act_quant(x, T)
+            pos, tok, _, off, tstart, mt = SM.route_sort(inds, E, TM)
+            h = SM.moe_mm(xq, R, gu[0], gu[1], gu[2], off, tstart, mt, 2 * Fi, 3, xscale=xs, tile=(TM, 64, 4), gather=tok)
+            hq, hs = SK.act_quant(h, R)
+            y = SM.moe_mm(hq, R, dn[0], dn[1], dn[2], off, tstart, mt, D, 1, xscale=hs, tile=(TM, 64, 4))
+            return SM.moe_combine(y, pos, scores, x, None, 0.0, T, quant=False)[0]
+
+        for _ in range(3):
+            moe_pass()
+        torch.cuda.synchronize()
+        reps_m = 20
+        e0.record(stream)
+        for _ in range(reps_m):
+            moe_pass()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps_m
+        ops = 2.0 * R * 3 * Fi * D
+        moe = {"workload": "BASELINE configs[3]: act quant + token sort + grouped gate_up GEMM (SwiGLU epilogue) + act "
+                           "quant + grouped down GEMM + weighted combine", "tokens": T, "experts": E, "topk": TOPK,
+               "ms": round(ms, 4), "tops": round(ops / ms / 1e9, 1),
+               "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
+        del gu, dn, x
+        torch.cuda.empty_cache()
+
     # ---- decode GEMV: achieved HBM GB/s, weights rotating beyond the cache -----------------------------------------
     decode = {}
     if not a.no_decode:
@@ -229,6 +306,8 @@ def main():
                                "down 2048x6144", "tokens": M_TOKENS, "weight_sets_rotated": n_sets},
         "pct_int8_peak": round(tops / PEAK_INT8_TOPS * 100, 2),
         "roofline": roofline,
+        "prefill_sweep": sweep,
+        "moe": moe,
         "decode": decode,
     }
     if not a.no_cpu:

@@ -140,7 +140,8 @@ int scmx_route_sort(const int32_t* inds, int M, int topk, int n_experts, int tm,
 /* Grouped W4A8 GEMM over expert segments: rows [off[e], off[e+1]) of the sorted activations use expert e's packed
  * weights (codes [E, N*K/8], bcodes [E, N, ..], wscale [E, N]).  When `gather` != NULL, sorted row r reads
  * xq[gather[r]] and xscale[gather[r]] (the xq[tok] gather of e2e/fused_olmoe.py:230 folded into the A-tile load);
- * otherwise xq / xscale are already in sorted order.  out: INT32 [R,N] (epi 0), T[R,N] (1), T[R,N/2] (3).
+ * otherwise xq / xscale are already in sorted order.  tm = 64, 128 or 256 is the row tile `tstart` was built for.
+ * out: INT32 [R,N] (epi 0), T[R,N] (1), T[R,N/2] (3).
  * Replaces moe_mm, e2e/sc_moe.py:19-92,169-185. */
 int scmx_moe_mm(const scmx_format* fmt, const int8_t* xq, const float* xscale, const int32_t* gather, int R,
                 const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const int32_t* off,

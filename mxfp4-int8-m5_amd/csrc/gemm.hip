@@ -592,8 +592,8 @@ static int moe_common(const char* who, const int8_t* xq, const float* xscale, co
         return SCMX_ERR_ARG;
     }
     if (int rc = check_gemm_common(who, R, N, K, epi, true, xq, xscale, wscale, nullptr, out)) return rc;
-    if (!off || !tstart || n_experts < 1 || !(tm == 64 || tm == 128)) {
-        set_error("%s: need off / tstart, n_experts >= 1 and a row tile of 64 or 128 (got %d)", who, tm);
+    if (!off || !tstart || n_experts < 1 || !(tm == 64 || tm == 128 || tm == 256)) {
+        set_error("%s: need off / tstart, n_experts >= 1 and a row tile of 64, 128 or 256 (got %d)", who, tm);
         return SCMX_ERR_ARG;
     }
     *a = GemmArgs{};
@@ -604,8 +604,10 @@ static int moe_common(const char* who, const int8_t* xq, const float* xscale, co
 
 static void launch_grouped(const GemmArgs& a, int bmode, int tm, hipStream_t s) {
     const int max_tiles = (a.M + tm - 1) / tm + a.n_experts;   // e2e/sc_moe.py:155
-    if (tm == 128)
-        launch_tile<128, 128, 128, 4, 2>(a, bmode, max_tiles, s);
+    if (tm == 256)
+        launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
+    else if (tm == 128)
+        launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
     else
         launch_tile<64, 128, 128, 2, 4>(a, bmode, max_tiles, s);
 }

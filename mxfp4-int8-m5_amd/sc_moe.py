@@ -49,7 +49,7 @@ def moe_mm(xq, R, codes, bcodes, wscale, off, tstart, max_tiles, N, epi, xscale=
            tile=(64, 64, 4), bk=128, gather=None, fmt=None):
     """Grouped W4A8 GEMM.  xq int8 [>= R, K] sorted by expert (or unsorted with gather=tok); packed expert weights
     codes [E, N*K/8], bcodes [E, N, ..], wscale f32 [E, N] -> INT32 [R, N] (EPI 0), bf16 [R, N] (1) or
-    bf16 [R, N/2] (3, interleaved gate/up).  tile[0] is the row tile the segments were built for (64 or 128)."""
+    bf16 [R, N/2] (3, interleaved gate/up).  tile[0] is the row tile the segments were built for (64, 128 or 256)."""
     fmt = fmt or F.DEFAULT
     K = xq.shape[1]
     E = wscale.shape[0]

@@ -45,7 +45,7 @@ def test_route_sort_contract(M, m, topk, e, tm):
     assert np.array_equal(host(o2), ro[3]) and np.array_equal(host(t2), ro[4]) and mt2 == mt
 
 
-@pytest.mark.parametrize("tm", [64, 128])
+@pytest.mark.parametrize("tm", [64, 128, 256])
 def test_grouped_gemm_uneven_segments(M, tm):
     """8 experts, 600 rows, experts 3 and 7 empty (e2e/sc_moe.py:213-215): INT32 exact, EPI 1 and 3 bit-exact,
     two-pass variant identical."""
