@@ -108,6 +108,11 @@ def mm_epi(xq, wq, xscale, wscale, epi, dtype=torch.bfloat16, res=None, deps=(),
     return _gemm(xq, wq, xscale, wscale, epi, res)
 
 
+def linear_w4a8_workspace(M, K):
+    """Bytes of workspace linear_w4a8 needs for M rows of K (the INT8 activations, then their scales)."""
+    return int(_lib.load().scmx_linear_w4a8_workspace(M, K))
+
+
 def linear_w4a8(x, codes, bcodes, wscale, N, epi=1, res=None, fmt=None, workspace=None):
     """One call for a whole W4A8 linear on bf16 activations [M, K]: the activation-quantization prologue and the
     fused-unpack GEMM are enqueued by a single C entry point (scmx_linear_w4a8).  Returns bf16 [M, N or N/2]."""

@@ -163,3 +163,21 @@ def test_bad_arguments_raise(S):
         S.mm_i8_i32(xq, wq)                      # K not a multiple of 128
     with pytest.raises(ValueError):
         S.act_quant(torch.zeros((4, 64), dtype=torch.bfloat16))   # CPU tensor
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (37, 64, 384), (300, 1024, 512), (700, 2048, 1152), (1100, 12288, 640)])
+def test_linear_one_call(S, m, n, k):
+    """linear_w4a8 (quantization prologue + GEMM behind one C entry point): ragged row counts, few and many column
+    tiles, a caller-provided workspace that ends up holding the INT8 rows and their scales."""
+    rng = np.random.default_rng(m + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k)
+    bits, x = llm_acts(rng, m, k)
+    xq_ref, xs_ref = linear.act_quant(x)
+    y_ref = linear.epilogue(linear.int_gemm(xq_ref, q), xs_ref, ws, 1)
+    work = torch.full((S.linear_w4a8_workspace(m, k),), 0x55, dtype=torch.uint8, device="cuda")
+    y = host(S.linear_w4a8(dev(bits), dev(codes), dev(bc), dev(ws), n, workspace=work))
+    assert np.array_equal(y, y_ref)
+    wh = host(work)
+    assert np.array_equal(wh[:m * k].view(np.int8).reshape(m, k), xq_ref)
+    off = (m * k + 255) & ~255
+    assert np.array_equal(wh[off:off + 4 * m].view(np.float32), xs_ref)
