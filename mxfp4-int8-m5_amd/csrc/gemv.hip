@@ -2,10 +2,13 @@
 //
 // Bandwidth-bound, so no MFMA: a wave owns R consecutive weight rows and walks K in steps of 64 blocks; each lane
 // loads 16 bytes of codes (one run of 32 weights) per row per step, so a wave reads 1 KiB of contiguous weights
-// per load instruction.  Codes are decoded to INT8 four at a time with byte-permute lookups and accumulated with
-// v_dot4_i32_i8 against the INT8 activations, which sit in LDS (one copy per workgroup, bytes of every 8-group
-// stored as elements 0,2,4,6,1,3,5,7 so the decode needs no re-interleave).  All sums are INT32, hence equal to the
-// GEMM's accumulators; the epilogues are the GEMM's.  `BATCH` activation rows share one pass over the weights.
+// per load instruction.  With one activation row the codes go through the FP4 conversion instruction (two codes ->
+// two half-precision values, sign and block scale included) and v_dot2c_f32_f16 against the activations staged in
+// LDS as half precision: all values are small integers, so the FP32 partial sums are exact.  With several rows, or
+// another weight format, codes are decoded to INT8 four at a time with byte-permute lookups and accumulated with
+// v_dot4_i32_i8 against INT8 activations in LDS (bytes of every 8-group stored as elements 0,2,4,6,1,3,5,7 so the
+// decode needs no re-interleave).  Either way the totals are the GEMM's INT32 accumulators and the epilogues are
+// the GEMM's.  `BATCH` activation rows share one pass over the weights.
 #include "scmx_common.h"
 
 namespace scmx {
@@ -34,8 +37,23 @@ __device__ __forceinline__ void store_perm8(int8_t* dst, const int q[8]) {
     *reinterpret_cast<u32x2*>(dst) = u32x2{e, o};
 }
 
-// Stage one activation row into LDS as permuted INT8 and return its scale.  `red` holds 66 floats.
-template <int NT>
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+
+// Eight INT8 codes as eight half-precision values (exact), in element order, 16 bytes.
+__device__ __forceinline__ void store_half8(int8_t* dst, const int q[8]) {
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const h2 p = h2{_Float16(float(q[2 * i])), _Float16(float(q[2 * i + 1]))};
+        o[i] = __builtin_bit_cast(uint32_t, p);
+    }
+    *reinterpret_cast<u32x4*>(dst) = o;
+}
+
+// Stage one activation row into LDS and return its scale: permuted INT8 (8 bytes per 8-group), or with F16 the codes
+// as half-precision values in element order (16 bytes per 8-group).  `red` holds 66 floats.
+template <int NT, bool F16>
 __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = a.K;
@@ -43,7 +61,14 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
         const u32x2* src = reinterpret_cast<const u32x2*>(reinterpret_cast<const int8_t*>(a.x) + size_t(row) * K);
         for (int c = tid; c < K / 8; c += NT) {
             const u32x2 v = src[c];
-            *reinterpret_cast<u32x2*>(sx + 8 * c) = u32x2{perm(v[1], v[0], 0x06040200u), perm(v[1], v[0], 0x07050301u)};
+            if (F16) {
+                int q[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = int(int8_t(v[i >> 2] >> (8 * (i & 3))));
+                store_half8(sx + 16 * c, q);
+            } else {
+                *reinterpret_cast<u32x2*>(sx + 8 * c) = u32x2{perm(v[1], v[0], 0x06040200u), perm(v[1], v[0], 0x07050301u)};
+            }
         }
         return a.xscale[row];
     }
@@ -112,7 +137,8 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
         int q[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], qi);
-        store_perm8(sx + 8 * c, q);
+        if (F16) store_half8(sx + 16 * c, q);
+        else store_perm8(sx + 8 * c, q);
     }
     __syncthreads();   // `red` is reused by the next row
     return s;
@@ -170,23 +196,23 @@ __device__ __forceinline__ int select_reduce(int (&v)[NV], int lane) {
     }
 }
 
-// Per-byte negation of INT8 bytes in -127..127.
-__device__ __forceinline__ uint32_t neg_i8x4(uint32_t x) {
-    const uint32_t n = ~x;
-    return ((n & 0x7F7F7F7Fu) + 0x01010101u) ^ (n & 0x80808080u);
-}
-
-template <int BATCH, int R, bool DEFAULT_FMT>
+// MODE 0: any format, byte-permute decode + v_dot4_i32_i8.  MODE 1: the published format with the same arithmetic
+// (lookup tables are constants).  MODE 2: the published format through the FP4 conversion
+// instruction: v_cvt_scalef32_pk_f16_fp4 turns two codes into two half-precision values, sign and block scale
+// included, and v_dot2c_f32_f16 multiplies them with the activations held as half precision.  Every value is an
+// integer below 2^11 and every partial sum one below 2^24, so the FP32 sums are exact and equal the integer ones.
+template <int BATCH, int R, int MODE>
 __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     constexpr int NT = 256;
     constexpr int NV = R * BATCH;
-    constexpr bool XSEL = DEFAULT_FMT && BATCH == 1;   // signs applied to the activations instead of the weights
+    constexpr bool DEFAULT_FMT = MODE != 0;
+    constexpr bool FP4 = MODE == 2;
+    constexpr int XB = FP4 ? 2 : 1;                    // bytes per staged activation
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int K = a.K, N = a.N;
-    int8_t* sx = smem;                                                   // [BATCH][K] permuted INT8 activations
+    int8_t* sx = smem;                                                   // [BATCH][K] staged activations
     const int Kp = (K + 2047) & ~2047;                                    // row pitch: whole 64-chunk slices, zero padded
-    int8_t* snx = smem + size_t(BATCH) * Kp;                             // XSEL: their negation
-    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * Kp * (XSEL ? 2 : 1));   // 68 floats + BATCH scales
+    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * Kp * XB);   // 68 floats + BATCH scales
     float* sxs = red + 68;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: row bases stay in scalar registers
@@ -198,22 +224,6 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         expert = (a.shared_expert >= 0 && slot == a.n_eidx) ? a.shared_expert : a.eidx[slot];
         xrow0 = slot * a.xstride;
     }
-#pragma unroll
-    for (int b = 0; b < BATCH; ++b) {
-        const float s = stage_row<NT>(a, xrow0 + b, sx + size_t(b) * Kp, red);
-        for (int c = K / 4 + tid; c < Kp / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
-        if (tid == 0) sxs[b] = s;
-    }
-    __syncthreads();
-    if (XSEL) {
-        for (int c = tid; c < Kp / 4; c += NT)
-            reinterpret_cast<uint32_t*>(snx)[c] = neg_i8x4(reinterpret_cast<const uint32_t*>(sx)[c]);
-        __syncthreads();
-    }
-
-    // constants kept in vector registers so that (x & k) | k' is one v_and_or_b32
-    uint32_t k_sign = 0x04040404u, k_ident = 0x03020100u;
-    asm volatile("" : "+v"(k_sign), "+v"(k_ident));
     const size_t erow = size_t(expert) * N;
     const int orow0 = a.eidx ? slot : 0;
     const int nchunk = K / 32;   // 16-byte code groups per row
@@ -250,15 +260,50 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         const uint32_t(&bc)[R] = it.bc;
         const uint8_t* brow = a.bcodes + (erow + size_t(g) * R) * a.bc_row_bytes;
         (void)brow;
-            u32x4 xv[BATCH][2], nxv[2];
+        if constexpr (FP4) {
+            float part[R][BATCH];
+            float scale[R];   // 2^(shift + 1): the codes are E2M1 values, the INT8 embedding is twice the value
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                scale[r] = __uint_as_float((128u + ((bc[r] >> (2 * (c & 3))) & 3u)) << 23);
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b) part[r][b] = 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                h8 xv[BATCH];   // the 8 activations of word j
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b)
+                    xv[b] = *reinterpret_cast<const h8*>(sx + (size_t(b) * Kp + 32u * c + 8u * j) * 2);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const uint32_t wj = w[r][j];
+                    const h2 q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 0);
+                    const h2 q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 1);
+                    const h2 q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 2);
+                    const h2 q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 3);
+#pragma unroll
+                    for (int b = 0; b < BATCH; ++b) {
+                        float p = part[r][b];
+                        p = __builtin_amdgcn_fdot2(q0, __builtin_shufflevector(xv[b], xv[b], 0, 1), p, false);
+                        p = __builtin_amdgcn_fdot2(q1, __builtin_shufflevector(xv[b], xv[b], 2, 3), p, false);
+                        p = __builtin_amdgcn_fdot2(q2, __builtin_shufflevector(xv[b], xv[b], 4, 5), p, false);
+                        p = __builtin_amdgcn_fdot2(q3, __builtin_shufflevector(xv[b], xv[b], 6, 7), p, false);
+                        part[r][b] = p;
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b) acc[r * BATCH + b] += int(part[r][b]);
+            return;
+        }
+            u32x4 xv[BATCH][2];
 #pragma unroll
             for (int b = 0; b < BATCH; ++b) {
                 xv[b][0] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * Kp + 32u * c);
                 xv[b][1] = *reinterpret_cast<const u32x4*>(sx + size_t(b) * Kp + 32u * c + 16);
-            }
-            if (XSEL) {
-                nxv[0] = *reinterpret_cast<const u32x4*>(snx + 32u * c);
-                nxv[1] = *reinterpret_cast<const u32x4*>(snx + 32u * c + 16);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -268,20 +313,6 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t wj = w[r][j];
-                    if (XSEL) {
-                        // magnitudes from the lookup; signs folded into a per-byte choice between x and -x:
-                        // selector byte i = i + 4 * sign picks byte i of x or of -x
-                        const uint32_t t = wj >> 4;
-                        const uint32_t me = perm(0x0C080604u, 0x03020100u, wj & 0x07070707u);
-                        const uint32_t mo = perm(0x0C080604u, 0x03020100u, t & 0x07070707u);
-                        const uint32_t xe = xv[0][j >> 1][2 * (j & 1)], xo = xv[0][j >> 1][2 * (j & 1) + 1];
-                        const uint32_t ne = nxv[j >> 1][2 * (j & 1)], no = nxv[j >> 1][2 * (j & 1) + 1];
-                        const uint32_t se = perm(ne, xe, ((wj >> 1) & k_sign) | k_ident);   // v_and_or_b32
-                        const uint32_t so = perm(no, xo, ((wj >> 5) & k_sign) | k_ident);
-                        part[0] = __builtin_amdgcn_sdot4(int(me), int(se), part[0], false);
-                        part[0] = __builtin_amdgcn_sdot4(int(mo), int(so), part[0], false);
-                        continue;
-                    }
                     uint32_t e, o;
                     if (DEFAULT_FMT) {
                         const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, 0u);   // folds to constants
@@ -365,36 +396,51 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         }
     };
 
-    int g = blockIdx.x * (NT / 64) + wave;
-    if (g >= groups) return;
-    int ci = 0;
+    // ---- driver ---------------------------------------------------------------------------------------------------
+    // Two register sets hold the wave's current and next item.  Both are requested before the activations are
+    // staged, so the first weights are already on their way while the workgroup quantizes its input.
+    const auto advance = [&](int& gi, int& cidx) {
+        if (++cidx == CI) {
+            cidx = 0;
+            gi += g_stride;
+        }
+    };
+    int g0 = blockIdx.x * (NT / 64) + wave, c0 = 0;   // item held by ia
+    int g1 = g0, c1 = 0;                              // item held by ib
+    advance(g1, c1);
+    Item ia, ib;
+    if (g0 < groups) load_item(ia, g0, lane + 64u * c0);
+    if (g1 < groups) load_item(ib, g1, lane + 64u * c1);
+
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+        const float s = stage_row<NT, FP4>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red);
+        for (int c = K * XB / 4 + tid; c < Kp * XB / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp * XB)[c] = 0u;
+        if (tid == 0) sxs[b] = s;
+    }
+    __syncthreads();
+    if (g0 >= groups) return;
     int acc[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) acc[i] = 0;
-    Item ia, ib;
-    load_item(ia, g, lane);
-    // one step: prefetch the next item into `nxt`, decode `cur`; returns false after the wave's last item
-    auto step = [&](const Item& cur, Item& nxt) {
-        int ng = g, nci = ci + 1;
-        if (nci == CI) {
-            nci = 0;
-            ng = g + g_stride;
-        }
-        const bool more = ng < groups;
-        load_item(nxt, more ? ng : g, lane + 64u * (more ? nci : ci));
-        compute_item(cur, g, lane + 64u * ci, acc);
-        if (ci == CI - 1) {
-            finish(g, acc);
+    // consume the item in `buf`, then refill `buf` with the item after the other set's
+    const auto work = [&](Item& buf, int& gi, int& cidx, int go, int co) {
+        compute_item(buf, gi, lane + 64u * cidx, acc);
+        if (cidx == CI - 1) {
+            finish(gi, acc);
 #pragma unroll
             for (int i = 0; i < NV; ++i) acc[i] = 0;
         }
-        g = ng;
-        ci = nci;
-        return more;
+        gi = go;
+        cidx = co;
+        advance(gi, cidx);
+        if (gi < groups) load_item(buf, gi, lane + 64u * cidx);
     };
     while (true) {
-        if (!step(ia, ib)) break;
-        if (!step(ib, ia)) break;
+        work(ia, g0, c0, g1, c1);
+        if (g1 >= groups) break;
+        work(ib, g1, c1, g0, c0);
+        if (g0 >= groups) break;
     }
 }
 
@@ -404,13 +450,20 @@ static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) 
     const int groups = a.N / R;
     const int want = (groups + 3) / 4;
     const int cap = max(1, 1024 / slots);
-    const dim3 grid(min(want, cap), slots), block(256);
-    const bool xsel = dflt && BATCH == 1;
-    const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (xsel ? 2 : 1) + (68 + BATCH) * sizeof(float);
-    if (dflt)
-        gemv_kernel<BATCH, R, true><<<grid, block, smem, s>>>(a);
-    else
-        gemv_kernel<BATCH, R, false><<<grid, block, smem, s>>>(a);
+    const int rounds = (want + cap - 1) / cap;                      // row groups each wave walks through
+    const dim3 grid((want + rounds - 1) / rounds, slots), block(256);   // ... the same number for every wave
+    // one activation row: the FP4-conversion path (activations staged as half precision) is the faster one; with
+    // more rows sharing the weight stream its extra LDS reads cost more than the integer dot products
+    const int mode = !dflt ? 0 : BATCH == 1 ? 2 : 1;
+    const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (mode == 2 ? 2 : 1) + (68 + BATCH) * sizeof(float);
+    auto go = [&](auto kernel) {
+        if (smem > 64 * 1024)
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
+        kernel<<<grid, block, smem, s>>>(a);
+    };
+    if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
+    else if (mode == 1) go(gemv_kernel<BATCH, R, 1>);
+    else go(gemv_kernel<BATCH, R, 0>);
 }
 
 template <int BATCH>
@@ -464,8 +517,8 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
         set_error("gemv: batch %d not in {1,2,4,8}", batch);
         return SCMX_ERR_ARG;
     }
-    if (size_t(batch) * ((K + 2047) & ~2047) * (batch == 1 ? 2 : 1) + 80 * sizeof(float) > 64 * 1024) {
-        set_error("gemv: batch * K = %zu bytes of activations exceed the 64 KiB staged per workgroup", size_t(batch) * K);
+    if (size_t(batch) * ((K + 2047) & ~2047) * 2 + 80 * sizeof(float) > 160 * 1024) {
+        set_error("gemv: batch * K = %zu activations exceed what one workgroup can stage (80 Ki)", size_t(batch) * K);
         return SCMX_ERR_ARG;
     }
     GemvArgs a = {};
