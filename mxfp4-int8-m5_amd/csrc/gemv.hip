@@ -397,20 +397,28 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     };
 
     // ---- driver ---------------------------------------------------------------------------------------------------
-    // Two register sets hold the wave's current and next item.  Both are requested before the activations are
-    // staged, so the first weights are already on their way while the workgroup quantizes its input.
+    // NB register sets hold the wave's current item and the NB - 1 after it.  All are requested before the
+    // activations are staged, so the first weights are already on their way while the workgroup quantizes its input.
+    constexpr int NB = 2;   // a third set costs occupancy and measured slower
     const auto advance = [&](int& gi, int& cidx) {
         if (++cidx == CI) {
             cidx = 0;
             gi += g_stride;
         }
     };
-    int g0 = blockIdx.x * (NT / 64) + wave, c0 = 0;   // item held by ia
-    int g1 = g0, c1 = 0;                              // item held by ib
-    advance(g1, c1);
-    Item ia, ib;
-    if (g0 < groups) load_item(ia, g0, lane + 64u * c0);
-    if (g1 < groups) load_item(ib, g1, lane + 64u * c1);
+    Item buf[NB];
+    int gq[NB], cq[NB];   // the item each set holds
+    gq[0] = blockIdx.x * (NT / 64) + wave;
+    cq[0] = 0;
+#pragma unroll
+    for (int i = 1; i < NB; ++i) {
+        gq[i] = gq[i - 1];
+        cq[i] = cq[i - 1];
+        advance(gq[i], cq[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+        if (gq[i] < groups) load_item(buf[i], gq[i], lane + 64u * cq[i]);
 
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
@@ -419,37 +427,39 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         if (tid == 0) sxs[b] = s;
     }
     __syncthreads();
-    if (g0 >= groups) return;
+    if (gq[0] >= groups) return;
     int acc[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) acc[i] = 0;
-    // consume the item in `buf`, then refill `buf` with the item after the other set's
-    const auto work = [&](Item& buf, int& gi, int& cidx, int go, int co) {
-        compute_item(buf, gi, lane + 64u * cidx, acc);
-        if (cidx == CI - 1) {
-            finish(gi, acc);
+    bool more = true;
+    while (more) {
 #pragma unroll
-            for (int i = 0; i < NV; ++i) acc[i] = 0;
+        for (int i = 0; i < NB; ++i) {   // consume set i, then refill it with the item after the newest one in flight
+            if (gq[i] >= groups) {
+                more = false;
+                break;
+            }
+            compute_item(buf[i], gq[i], lane + 64u * cq[i], acc);
+            if (cq[i] == CI - 1) {
+                finish(gq[i], acc);
+#pragma unroll
+                for (int v = 0; v < NV; ++v) acc[v] = 0;
+            }
+            gq[i] = gq[(i + NB - 1) % NB];
+            cq[i] = cq[(i + NB - 1) % NB];
+            advance(gq[i], cq[i]);
+            if (gq[i] < groups) load_item(buf[i], gq[i], lane + 64u * cq[i]);
         }
-        gi = go;
-        cidx = co;
-        advance(gi, cidx);
-        if (gi < groups) load_item(buf, gi, lane + 64u * cidx);
-    };
-    while (true) {
-        work(ia, g0, c0, g1, c1);
-        if (g1 >= groups) break;
-        work(ib, g1, c1, g0, c0);
-        if (g0 >= groups) break;
     }
 }
 
 template <int BATCH, int R>
 static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
-    // enough workgroups to fill the chip (4 waves each), but no more than ~16 resident waves per CU: waves loop
+    // enough workgroups to fill the chip (4 waves each), but no more than the ~24 waves per CU that can be resident:
+    // waves loop
     const int groups = a.N / R;
     const int want = (groups + 3) / 4;
-    const int cap = max(1, 1024 / slots);
+    const int cap = max(1, 1536 / slots);
     const int rounds = (want + cap - 1) / cap;                      // row groups each wave walks through
     const dim3 grid((want + rounds - 1) / rounds, slots), block(256);   // ... the same number for every wave
     // one activation row: the FP4-conversion path (activations staged as half precision) is the faster one; with
