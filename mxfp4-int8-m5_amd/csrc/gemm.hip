@@ -207,8 +207,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                         if (w * NKK / WPC != q) continue;
                         if (BMODE == B_PACKED_DEFAULT) {
                             const uint32_t blk = uint32_t(k0 + b_k[j]) >> 5;
-                            const BlockLut t = scaled_lut_shift(0x03020100u, 0x0C080604u, (uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u);
-                            decode_word(r.b[j][w], t, o[j][2 * w], o[j][2 * w + 1]);
+                            decode_word_fp4(r.b[j][w], fp4_scale((uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u), o[j][2 * w],
+                                            o[j][2 * w + 1]);
                         } else {
                             const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> a.fmt.block_log2;
                             const uint32_t bc = block_code(a.bcodes + erow * a.bc_row_bytes + b_bc[j], blk, a.fmt.bc_bits);

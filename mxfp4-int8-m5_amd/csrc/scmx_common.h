@@ -132,6 +132,23 @@ __device__ __forceinline__ void decode_word_split(uint32_t w, const BlockLut& t,
     o = decode4(w >> 4, t);
 }
 
+// The published format (E2M1 codes, power-of-two block multipliers) through the FP4 conversion instruction:
+// v_cvt_scalef32_pk_f16_fp4 turns the two codes of one byte into two half-precision values, sign included, times a
+// power-of-two scale; with scale = 2^(shift + 1) these are the INT8 embedding q (|q| <= 96) exactly.  Adding 1536
+// puts q into the low mantissa bits (1536 + q lies in [1024, 2048), where half precision steps by 1), so the low
+// byte of each half is q in two's complement; one byte permute gathers four of them.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float fp4_scale(uint32_t shift) { return __uint_as_float((128u + shift) << 23); }
+__device__ __forceinline__ void decode_word_fp4(uint32_t w, float scale, uint32_t& a, uint32_t& b) {
+    const half2_t bias = half2_t{_Float16(1536.0f), _Float16(1536.0f)};
+    const half2_t q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 0) + bias;
+    const half2_t q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 1) + bias;
+    const half2_t q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 2) + bias;
+    const half2_t q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 3) + bias;
+    a = perm(__builtin_bit_cast(uint32_t, q1), __builtin_bit_cast(uint32_t, q0), 0x06040200u);
+    b = perm(__builtin_bit_cast(uint32_t, q3), __builtin_bit_cast(uint32_t, q2), 0x06040200u);
+}
+
 // Block code of block `blk` in a row whose block codes start at `row_bc`.
 __device__ __forceinline__ uint32_t block_code(const uint8_t* row_bc, uint32_t blk, int bc_bits) {
     const uint32_t per_byte = 8u / bc_bits;
