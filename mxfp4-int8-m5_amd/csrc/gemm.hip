@@ -481,8 +481,8 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     const long cus = 256;
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
     if (tiles(256, 128) >= cus) return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
+    if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
     if (tiles(256, 64) >= cus) return launch_tile<256, 64, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
-    if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
     if (tiles(128, 64) >= cus) return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
     return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
 }
