@@ -119,7 +119,8 @@ int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn,
 
 /* ---- decode --------------------------------------------------------------------------------------------------- */
 
-/* W4A8 GEMV on packed weights, `batch` input rows sharing one weight stream (batch 1..8; the reference has batch 1).
+/* W4A8 GEMV on packed weights, `batch` input rows sharing one weight stream (batch 1, 2, 4 or 8; the reference has
+ * batch 1).
  *   pro 0: xq int8 [batch, K] + xscale [batch];  pro 1: x T[batch, K] quantized in the kernel;
  *   pro 2: RMSNorm(x, nw, eps) then INT8 in the kernel.
  *   eidx != NULL (MoE): `slots` output rows, slot j uses expert eidx[j] (or `shared_expert` for the slot after the
