@@ -117,12 +117,28 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
             }
         }
     };
+    // Rows of up to 8 * NT * KEEP values are read once and kept in registers between the maximum and the rounding.
+    constexpr int KEEP = 1;   // more would cost the kernel a wave of occupancy (the first weight loads are in flight too)
+    const bool keep = K <= 8 * NT * KEEP;
+    float kept[KEEP][8];
     float amax = 0.0f;
-    for (int c = tid; c < K / 8; c += NT) {
-        float v[8];
-        values(c, v);
+    if (keep) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+        for (int j = 0; j < KEEP; ++j) {
+            const int c = tid + j * NT;
+            if (c < K / 8) {
+                values(c, kept[j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(kept[j][i]));
+            }
+        }
+    } else {
+        for (int c = tid; c < K / 8; c += NT) {
+            float v[8];
+            values(c, v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+        }
     }
     amax = wave_max(amax);
     if (lane == 0) red[wave] = amax;
@@ -131,14 +147,25 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
     for (int w = 0; w < NT / 64; ++w) amax = fmaxf(amax, red[w]);
     const float s = __fdiv_rn(amax, 127.0f);
     const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
-    for (int c = tid; c < K / 8; c += NT) {
-        float v[8];
-        values(c, v);
+    const auto emit = [&](int c, const float (&v)[8]) {
         int q[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], qi);
         if (F16) store_half8(sx + 16 * c, q);
         else store_perm8(sx + 8 * c, q);
+    };
+    if (keep) {
+#pragma unroll
+        for (int j = 0; j < KEEP; ++j) {
+            const int c = tid + j * NT;
+            if (c < K / 8) emit(c, kept[j]);
+        }
+    } else {
+        for (int c = tid; c < K / 8; c += NT) {
+            float v[8];
+            values(c, v);
+            emit(c, v);
+        }
     }
     __syncthreads();   // `red` is reused by the next row
     return s;
