@@ -1,6 +1,7 @@
 // Decode GEMV on packed SC-MXFP4 weights: y[b, n] = epi(xs[b] * ws[n] * sum_k xq[b, k] * q[n, k]).
 //
-// Bandwidth-bound, so no MFMA: a wave owns R consecutive weight rows and walks K in steps of 64 blocks; each lane
+// One activation row is bandwidth-bound and needs no MFMA: a wave owns R consecutive weight rows and walks K in steps
+// of 64 blocks; each lane
 // loads 16 bytes of codes (one run of 32 weights) per row per step, so a wave reads 1 KiB of contiguous weights
 // per load instruction.  With one activation row the codes go through the FP4 conversion instruction (two codes ->
 // two half-precision values, sign and block scale included) and v_dot2c_f32_f16 against the activations staged in
@@ -8,7 +9,9 @@
 // another weight format, codes are decoded to INT8 four at a time with byte-permute lookups and accumulated with
 // v_dot4_i32_i8 against INT8 activations in LDS (bytes of every 8-group stored as elements 0,2,4,6,1,3,5,7 so the
 // decode needs no re-interleave).  Either way the totals are the GEMM's INT32 accumulators and the epilogues are
-// the GEMM's.  `BATCH` activation rows share one pass over the weights.
+// the GEMM's.  `BATCH` activation rows share one pass over the weights; for the published format they go through
+// gemv_mfma_kernel below, which hands the dot products to the 4x4x4 INT8 MFMA so that the vector work per weight
+// does not grow with the number of rows.
 #include "scmx_common.h"
 
 namespace scmx {
@@ -51,10 +54,21 @@ __device__ __forceinline__ void store_half8(int8_t* dst, const int q[8]) {
     *reinterpret_cast<u32x4*>(dst) = o;
 }
 
+// Eight INT8 codes in element order, 8 bytes.
+__device__ __forceinline__ void store_plain8(int8_t* dst, const int q[8]) {
+    u32x2 o = u32x2{0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i >> 2] |= (uint32_t(q[i]) & 0xFFu) << (8 * (i & 3));
+    *reinterpret_cast<u32x2*>(dst) = o;
+}
+
+enum { X_PERM8 = 0, X_HALF = 1, X_PLAIN8 = 2 };
+
 // Stage one activation row into LDS and return its scale: permuted INT8 (8 bytes per 8-group), or with F16 the codes
 // as half-precision values in element order (16 bytes per 8-group).  `red` holds 66 floats.
-template <int NT, bool F16>
+template <int NT, int XMODE>
 __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
+    constexpr bool F16 = XMODE == X_HALF;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = a.K;
     if (a.pro == 0) {
@@ -66,6 +80,8 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) q[i] = int(int8_t(v[i >> 2] >> (8 * (i & 3))));
                 store_half8(sx + 16 * c, q);
+            } else if (XMODE == X_PLAIN8) {
+                *reinterpret_cast<u32x2*>(sx + 8 * c) = v;
             } else {
                 *reinterpret_cast<u32x2*>(sx + 8 * c) = u32x2{perm(v[1], v[0], 0x06040200u), perm(v[1], v[0], 0x07050301u)};
             }
@@ -152,6 +168,7 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], qi);
         if (F16) store_half8(sx + 16 * c, q);
+        else if (XMODE == X_PLAIN8) store_plain8(sx + 8 * c, q);
         else store_perm8(sx + 8 * c, q);
     };
     if (keep) {
@@ -449,7 +466,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-        const float s = stage_row<NT, FP4>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red);
+        const float s = stage_row<NT, FP4 ? X_HALF : X_PERM8>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red);
         for (int c = K * XB / 4 + tid; c < Kp * XB / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp * XB)[c] = 0u;
         if (tid == 0) sxs[b] = s;
     }
@@ -480,6 +497,154 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     }
 }
 
+// Several activation rows against the published format: the dot products go to the matrix pipe.
+// v_mfma_i32_4x4x4_16b_i8 multiplies, in each of 16 blocks of 4 lanes, a 4x4 INT8 matrix of activations (lane i of the
+// block: 4 consecutive k of activation row i) with one of weights (lane j: the same 4 k of weight row j) and adds the
+// 4x4 INT32 result (lane j, register r = activation row r, weight row j).  A wave owns 4 consecutive weight rows;
+// lane (block b, j) loads four 16-byte runs of row j (chunks b, b+16, b+32, b+48 of the 64-chunk slice), decodes
+// them with the FP4 conversion and feeds 8 MFMAs per run; the 16 blocks cover different k, so a row group ends with a
+// sum over the blocks.  Vector work per weight no longer grows with the number of activation rows.
+template <int BATCH>
+__global__ __launch_bounds__(256) void gemv_mfma_kernel(const GemvArgs a) {
+    constexpr int NT = 256;
+    constexpr int NSET = BATCH > 4 ? 2 : 1;    // MFMA accumulators: activation rows 0..3 and 4..7
+    constexpr int XR = 4 * NSET;               // activation rows as the MFMA sees them (zero rows pad BATCH up)
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    const int K = a.K, N = a.N;
+    const int Kp = (K + 2047) & ~2047;
+    int8_t* sx = smem;                                                   // [XR][Kp] INT8 in element order
+    float* red = reinterpret_cast<float*>(smem + size_t(XR) * Kp);      // 68 floats + BATCH scales
+    float* sxs = red + 68;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int blk = lane >> 2, j = lane & 3;
+    const int nchunk = K / 32, groups = N / 4;
+    const int CI = (nchunk + 63) / 64;
+    const int g_stride = gridDim.x * (NT / 64);
+
+    struct Item {
+        u32x4 w[4];   // runs blk, blk + 16, blk + 32, blk + 48 of the slice, weight row j
+        u32x4 bc;     // the slice's 16 block-code bytes of row j
+    };
+    const auto load_item = [&](Item& it, int g, int ci) {
+        const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + size_t(g) * 4 * (K / 2);   // uniform
+        const uint8_t* brow = a.bcodes + size_t(g) * 4 * a.bc_row_bytes;
+        const __amdgpu_buffer_rsrc_t rc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(crow), 0, 4 * (K / 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rb =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(brow), 0, 4 * a.bc_row_bytes, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = min(ci * 64 + blk + 16 * i, nchunk - 1);   // past the row: any valid run (its activations are 0)
+            it.w[i] = __builtin_amdgcn_raw_buffer_load_b128(rc, j * (K / 2) + 16 * c, 0, 0);
+        }
+        it.bc = __builtin_amdgcn_raw_buffer_load_b128(rb, j * a.bc_row_bytes, ci * 16, 0);   // out of range reads 0
+    };
+    v4i acc[NSET], acc2[NSET];   // two accumulation chains per set: consecutive MFMAs do not wait for each other
+    const auto compute_item = [&](const Item& it, int ci) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t c = uint32_t(ci * 64 + blk + 16 * i);
+            // block code of run c: byte blk / 4 of dword i of the slice's 16 bytes, bits 2 * (blk % 4)
+            const float scale = fp4_scale((it.bc[i] >> (2 * blk)) & 3u);
+            u32x4 xv[NSET][2];
+#pragma unroll
+            for (int s = 0; s < NSET; ++s) {
+                xv[s][0] = *reinterpret_cast<const u32x4*>(sx + size_t(4 * s + j) * Kp + 32u * c);
+                xv[s][1] = *reinterpret_cast<const u32x4*>(sx + size_t(4 * s + j) * Kp + 32u * c + 16);
+            }
+#pragma unroll
+            for (int wd = 0; wd < 4; ++wd) {
+                uint32_t qa, qb;
+                decode_word_fp4(it.w[i][wd], scale, qa, qb);
+#pragma unroll
+                for (int s = 0; s < NSET; ++s) {
+                    acc[s] = __builtin_amdgcn_mfma_i32_4x4x4i8(int(xv[s][wd >> 1][2 * (wd & 1)]), int(qa), acc[s], 0, 0, 0);
+                    acc2[s] = __builtin_amdgcn_mfma_i32_4x4x4i8(int(xv[s][wd >> 1][2 * (wd & 1) + 1]), int(qb), acc2[s], 0, 0, 0);
+                }
+            }
+        }
+    };
+    const auto finish = [&](int g) {
+        // Totals over the 16 blocks (lane bits 2..5).  The first exchange steps also halve the set of values a lane
+        // carries, so a lane ends with one total: that of activation row `brow`, weight row j.
+        constexpr int NV = 4 * NSET;
+        int vals[NV];
+#pragma unroll
+        for (int s = 0; s < NSET; ++s)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vals[4 * s + r] = acc[s][r] + acc2[s][r];
+        const int tot = select_reduce<NV, 4>(vals, lane);
+        const int brow = NSET == 1 ? 2 * (blk & 1) + ((blk >> 1) & 1)
+                                   : 4 * (blk & 1) + 2 * ((blk >> 1) & 1) + ((blk >> 2) & 1);
+        const bool emit = brow < BATCH && (blk >> (NSET == 1 ? 2 : 3)) == 0;   // one of the lanes that hold this total
+        const int n = g * 4 + j;
+        float y = 0.0f;
+        if (emit) y = __fmul_rn(__fmul_rn(float(tot), sxs[brow]), a.wscale[n]);
+        if (a.epi == SCMX_EPI_SWIGLU) {   // rows (g, g, u, u): lanes j = 0, 1 pair with j + 2
+            const float yb = round_bf16(y);
+            const float up = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(yb), 0x4E, 0xF, 0xF, false));
+            if (emit && j < 2) a.out[size_t(brow) * (N / 2) + (g * 4) / 2 + j] = swiglu_bf16(yb, up);
+        } else if (emit) {
+            const size_t o = size_t(brow) * N + n;
+            if (a.epi == SCMX_EPI_SCALE) a.out[o] = f32_to_bf16(y);
+            else a.out[o] = f32_to_bf16(__fadd_rn(bf16_to_f32(a.res[o]), round_bf16(y)));
+        }
+    };
+
+    const auto advance = [&](int& gi, int& cidx) {
+        if (++cidx == CI) {
+            cidx = 0;
+            gi += g_stride;
+        }
+    };
+    Item buf[2];
+    int gq[2], cq[2];
+    gq[0] = blockIdx.x * (NT / 64) + wave;
+    cq[0] = 0;
+    gq[1] = gq[0];
+    cq[1] = 0;
+    advance(gq[1], cq[1]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        if (gq[i] < groups) load_item(buf[i], gq[i], cq[i]);
+
+#pragma unroll
+    for (int b = 0; b < XR; ++b) {
+        if (b < BATCH) {
+            const float s = stage_row<NT, X_PLAIN8>(a, b, sx + size_t(b) * Kp, red);
+            for (int c = K / 4 + tid; c < Kp / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
+            if (tid == 0) sxs[b] = s;
+        } else {
+            for (int c = tid; c < Kp / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
+        }
+    }
+    __syncthreads();
+    if (gq[0] >= groups) return;
+#pragma unroll
+    for (int s = 0; s < NSET; ++s) acc[s] = acc2[s] = v4i{0, 0, 0, 0};
+    bool more = true;
+    while (more) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            if (gq[i] >= groups) {
+                more = false;
+                break;
+            }
+            compute_item(buf[i], cq[i]);
+            if (cq[i] == CI - 1) {
+                finish(gq[i]);
+#pragma unroll
+                for (int s = 0; s < NSET; ++s) acc[s] = acc2[s] = v4i{0, 0, 0, 0};
+            }
+            gq[i] = gq[1 - i];
+            cq[i] = cq[1 - i];
+            advance(gq[i], cq[i]);
+            if (gq[i] < groups) load_item(buf[i], gq[i], cq[i]);
+        }
+    }
+}
+
 template <int BATCH, int R>
 static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
     // enough workgroups to fill the chip (4 waves each), but no more than the ~24 waves per CU that can be resident:
@@ -504,7 +669,22 @@ static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) 
 }
 
 template <int BATCH>
+static void launch_gemv_mfma(const GemvArgs& a, hipStream_t s) {
+    const int groups = a.N / 4;
+    const int want = (groups + 3) / 4;
+    const int rounds = (want + 1279) / 1280;   // 5 waves per SIMD are resident
+    const dim3 grid((want + rounds - 1) / rounds), block(256);
+    const size_t smem = size_t(BATCH > 4 ? 8 : 4) * ((a.K + 2047) & ~2047) + (68 + BATCH) * sizeof(float);
+    if (smem > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mfma_kernel<BATCH>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
+    gemv_mfma_kernel<BATCH><<<grid, block, smem, s>>>(a);
+}
+
+template <int BATCH>
 static void launch_gemv_rows(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
+    if (BATCH > 1 && dflt && !a.eidx && a.N % 4 == 0 && a.K % 512 == 0)
+        return launch_gemv_mfma<BATCH>(a, s);
     // more rows per wave = more loads in flight per lane; fewer = more waves for narrow layers
     const long rows = long(a.N) * slots;
     constexpr int RMAX = BATCH == 1 ? 4 : BATCH == 2 ? 4 : BATCH == 4 ? 2 : 1;   // keeps several waves per SIMD resident

@@ -102,6 +102,28 @@ def test_gemv_batch_equals_rows(G, batch):
     assert np.array_equal(yp, linear.gemv(rq, rs, q, ws, 1))
 
 
+@pytest.mark.parametrize("batch,n,k", [(2, 512, 512), (4, 2048, 6144), (8, 256, 1536), (4, 1028, 1024), (4, 1022, 1024),
+                                       (4, 512, 640)])
+def test_gemv_batch_shapes_and_epilogues(G, batch, n, k):
+    """Several rows per pass over K of one, several and fractional 2048-slices, N off the 4-row grain, K off the
+    512 grain, with the residual and SwiGLU epilogues."""
+    rng = np.random.default_rng(batch + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k)
+    xq = rng.integers(-127, 128, (batch, k)).astype(np.int8)
+    xq[0, :16] = 127
+    xs = (np.abs(rng.standard_normal(batch)) * 1e-2 + 1e-3).astype(F32)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    ref1 = linear.gemv(xq, xs, q, ws, 1)
+    assert np.array_equal(host(G.gemv(dev(xq), dc, db, dev(xs), dw, n, 1)), ref1)
+    res = bf16.to_bits(rng.standard_normal((batch, n)).astype(F32))
+    assert np.array_equal(host(G.gemv(dev(xq), dc, db, dev(xs), dw, n, 2, res=dev(res))), linear.gemv(xq, xs, q, ws, 2, res))
+    if n % 4 == 0:
+        perm = linear.interleave_gate_up(n // 2)
+        cp = codes.reshape(n, -1)[perm].reshape(-1)
+        y3 = host(G.gemv(dev(xq), dev(cp), dev(bc[perm]), dev(xs), dev(ws[perm]), n, 3))
+        assert np.array_equal(y3, linear.swiglu(ref1[:, :n // 2], ref1[:, n // 2:]))
+
+
 def test_gemv_expert_gather(G):
     """MoE: slot j uses expert eidx[j] and its own input row; `shared` appends one more slot
     (e2e/sc_decode.py:292-307, e2e/decode.py:126-143)."""
