@@ -449,7 +449,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             }
         }
         if (c + epp <= on)
-            *reinterpret_cast<u32x4*>(dst) = v;
+            // streaming store: the tile is not read again by this kernel, and lines that never sit dirty in the L2
+            // do not have to be written back when the kernel ends
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
         else   // the row ends inside this piece: rows are multiples of 4 elements, so exactly half of it is valid
             *reinterpret_cast<u32x2*>(dst) = u32x2{v[0], v[1]};
     }
