@@ -280,6 +280,94 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const int32_t* __restr
     for (int p = R + tid; p < R + tm; p += 1024) tok[p] = 0;   // padding rows gather token 0
 }
 
+// ---- MoE: the same counting sort over several workgroups, three launches -------------------------------------------
+// Workgroup g owns assignments [g * 1024, (g + 1) * 1024), the last one also the tail of fewer than 1024.  Its
+// per-expert counts, and later its per-expert first rows, are parked in pos[g * 1024 + e] (E <= 1024), i.e. inside the
+// part of `pos` that only this workgroup writes in the last pass, so no extra memory is needed and no workgroup reads
+// what another one may already have overwritten.
+constexpr int RS_CHUNK = 1024;
+
+__global__ __launch_bounds__(RS_CHUNK) void route_count_kernel(const int32_t* __restrict__ inds, int R, int E,
+                                                               int32_t* __restrict__ pos) {
+    __shared__ uint32_t cnt[1024];
+    const int tid = threadIdx.x;
+    const int end = blockIdx.x == gridDim.x - 1 ? R : (blockIdx.x + 1) * RS_CHUNK;   // the last one takes the tail
+    cnt[tid] = 0;
+    __syncthreads();
+    for (int i = blockIdx.x * RS_CHUNK + tid; i < end; i += RS_CHUNK) atomicAdd(&cnt[min(max(inds[i], 0), E - 1)], 1u);
+    __syncthreads();
+    if (tid < E) pos[blockIdx.x * RS_CHUNK + tid] = int32_t(cnt[tid]);
+}
+
+// One workgroup: thread e turns the G counts of expert e into exclusive prefixes (the rows of the expert taken by
+// earlier workgroups), then the experts' totals are scanned into off / tstart as in the single-workgroup kernel.
+__global__ __launch_bounds__(1024) void route_scan_kernel(int G, int E, int tm, int32_t* __restrict__ pos,
+                                                          int32_t* __restrict__ off, int32_t* __restrict__ tstart) {
+    __shared__ uint32_t cur[1024], tl[1024];
+    const int tid = threadIdx.x;
+    uint32_t c = 0;
+    if (tid < E) {
+        int g = 0;
+        for (; g + 8 <= G; g += 8) {
+            uint32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = uint32_t(pos[(g + u) * RS_CHUNK + tid]);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                pos[(g + u) * RS_CHUNK + tid] = int32_t(c);
+                c += v[u];
+            }
+        }
+        for (; g < G; ++g) {
+            const uint32_t v = uint32_t(pos[g * RS_CHUNK + tid]);
+            pos[g * RS_CHUNK + tid] = int32_t(c);
+            c += v;
+        }
+    }
+    uint32_t so = c, st = (c + tm - 1) / tm;
+    const uint32_t t0 = st;
+    cur[tid] = so;
+    tl[tid] = st;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const uint32_t ao = tid >= d ? cur[tid - d] : 0u, at = tid >= d ? tl[tid - d] : 0u;
+        __syncthreads();
+        so += ao;
+        st += at;
+        cur[tid] = so;
+        tl[tid] = st;
+        __syncthreads();
+    }
+    if (tid < E) {
+        off[tid] = int32_t(so - c);
+        tstart[tid] = int32_t(st - t0);
+    }
+    if (tid == E - 1) {
+        off[E] = int32_t(so);
+        tstart[E] = int32_t(st);
+    }
+}
+
+__global__ __launch_bounds__(RS_CHUNK) void route_place_kernel(const int32_t* __restrict__ inds, int R, int topk, int E,
+                                                               int tm, const int32_t* __restrict__ off,
+                                                               int32_t* __restrict__ pos, int32_t* __restrict__ tok,
+                                                               int32_t* __restrict__ esorted) {
+    __shared__ uint32_t cur[1024];
+    const int tid = threadIdx.x;
+    const int end = blockIdx.x == gridDim.x - 1 ? R : (blockIdx.x + 1) * RS_CHUNK;
+    if (tid < E) cur[tid] = uint32_t(off[tid]) + uint32_t(pos[blockIdx.x * RS_CHUNK + tid]);
+    __syncthreads();   // the parked prefixes are in LDS before any pos[i] of this range is written
+    for (int i = blockIdx.x * RS_CHUNK + tid; i < end; i += RS_CHUNK) {
+        const int e = min(max(inds[i], 0), E - 1);
+        const uint32_t p = atomicAdd(&cur[e], 1u);
+        pos[i] = int32_t(p);
+        tok[p] = i / topk;
+        esorted[p] = e;
+    }
+    if (blockIdx.x == 0)
+        for (int p = R + tid; p < R + tm; p += RS_CHUNK) tok[p] = 0;   // padding rows gather token 0
+}
+
 // ---- MoE: weighted combine of the top-k expert outputs, sequential in bf16 ---------------------------------------
 __global__ __launch_bounds__(NT) void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ pos,
                                                          const uint16_t* __restrict__ scores, const uint16_t* __restrict__ sscore,
@@ -410,8 +498,20 @@ int scmx_route_sort(const int32_t* inds, int M, int topk, int n_experts, int tm,
         set_error("route_sort: null pointer, or n_experts (%d) outside 1..1024", n_experts);
         return SCMX_ERR_ARG;
     }
-    route_sort_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>(inds, M * topk, topk, n_experts, tm, pos, tok,
-                                                                        esorted, off, tstart);
+    const long long R = (long long)M * topk;
+    if (R > 0x7FFFFFFF - tm) {
+        set_error("route_sort: M * topk = %lld beyond 32-bit row indices", R);
+        return SCMX_ERR_ARG;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int G = int(R / RS_CHUNK);   // whole chunks; the last workgroup also takes the tail
+    if (G < 4) {   // small inputs: one launch of one workgroup beats three launches
+        route_sort_kernel<<<dim3(1), dim3(1024), 0, st>>>(inds, int(R), topk, n_experts, tm, pos, tok, esorted, off, tstart);
+        return check_launch("route_sort");
+    }
+    route_count_kernel<<<dim3(G), dim3(RS_CHUNK), 0, st>>>(inds, int(R), n_experts, pos);
+    route_scan_kernel<<<dim3(1), dim3(1024), 0, st>>>(G, n_experts, tm, pos, off, tstart);
+    route_place_kernel<<<dim3(G), dim3(RS_CHUNK), 0, st>>>(inds, int(R), topk, n_experts, tm, off, pos, tok, esorted);
     return check_launch("route_sort");
 }
 

@@ -30,7 +30,7 @@ def skewed_routing(rng, tokens, experts, topk):
 
 
 @pytest.mark.parametrize("m,topk,e,tm", [(75, 8, 8, 64), (4096, 8, 64, 128), (2048, 9, 257, 64), (1, 8, 64, 64),
-                                         (300, 1, 1024, 128)])
+                                         (300, 1, 1024, 128), (1000, 5, 1024, 64), (515, 8, 300, 128)])
 def test_route_sort_contract(M, m, topk, e, tm):
     rng = np.random.default_rng(m + e)
     inds, _ = skewed_routing(rng, m, e, topk)
