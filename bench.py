@@ -86,6 +86,7 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV leg")
     ap.add_argument("--no-moe", action="store_true", help="skip the grouped mixture-of-experts leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 512 / 8192 prefill sweep")
+    ap.add_argument("--no-quant", action="store_true", help="skip the device quantizer leg")
     ap.add_argument("--profile-copy", action="store_true",
                     help="first run one plain 256 MiB device copy: the known-size kernel that calibrates FETCH_SIZE / "
                          "WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -296,6 +297,37 @@ def main():
             del wsets
             torch.cuda.empty_cache()
 
+    # ---- offline quantizer on the device: float32 weights -> packed SC-MXFP4 -----------------------------------
+    quant = {}
+    if not a.no_quant:
+        torch.cuda.empty_cache()
+        n, k = 12288, 2048
+        wf = torch.randn((n, k), device=dev) * 0.02
+        qc = torch.empty(n * k // 8, dtype=torch.int32, device=dev)
+        qb = torch.empty((n, k // 128), dtype=torch.uint8, device=dev)
+        qw = torch.empty(n, dtype=torch.float32, device=dev)
+        qargs = (wf.data_ptr(), 0, n, k, 32, qc.data_ptr(), qb.data_ptr(), qw.data_ptr(), sp)
+        for _ in range(2):
+            check(lib.scmx_quantize_sc(*qargs))
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(10):
+            check(lib.scmx_quantize_sc(*qargs))
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / 10 * 1e3
+        quant = {"workload": f"float32 {n}x{k} -> codes + block codes + row scales (exponent search over 3 candidates "
+                             "in float64, bit-identical to the host quantizer)", "us": round(us, 1),
+                 "gweights_per_s": round(n * k / us / 1e3, 2),
+                 "gbps": round(n * k * (2 * 4 + 0.5 + 1.0 / 128) / us / 1e3, 1)}   # the row is read twice
+        if not a.no_cpu:
+            from oracle import layout as olayout
+            wh = wf[:256].cpu().numpy().astype(np.float64)
+            t0 = time.perf_counter()
+            olayout.quantize(wh)
+            quant["cpu_oracle_gweights_per_s"] = round(256 * k / (time.perf_counter() - t0) / 1e9, 4)
+        del wf, qc, qb, qw
+
     result = {
         "metric": "INT8 TOPS, W4A8 prefill GEMM M=2048 (Qwen3-1.7B layer shapes), 1 GPU; decode GEMV GB/s alongside",
         "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -309,6 +341,7 @@ def main():
         "prefill_sweep": sweep,
         "moe": moe,
         "decode": decode,
+        "quantize": quant,
     }
     if not a.no_cpu:
         result["cpu_baseline"] = cpu_baseline()

@@ -170,6 +170,18 @@ int scmx_moe_combine(const uint16_t* y, const int32_t* pos, const uint16_t* scor
 int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,
                      void* stream);
 
+/* ---- offline quantizer ------------------------------------------------------------------------------------------ */
+
+/* Float weights w [N, K] (float32, or bf16 when w_is_bf16 != 0) -> SC-MXFP4 in the packed layout with `block`-wide
+ * blocks (32 = the published format, 16 = its 16-block power-of-two sibling): codes u32 [N*K/8], bcodes u8
+ * [N, K/(4*block)] (2-bit shifts), wscale f32 [N] = 2^(E_lo - 1).  Per block the exponent floor(log2 amax) - 2 is
+ * tried against its two neighbours (-1 first, then +1, strict improvement of the float64 squared error), rows are
+ * constrained to an exponent spread of 3, values are rounded to E2M1 with ties to the lower magnitude.  Bit-identical
+ * to the host procedure: sim/mx_int8.py:39-109 (block_exponents "search", constrain_spread, dequant_mx, embed_int8),
+ * sim/make_testcase.py:26-44 (pack), e2e/sc_format.py:105-111 (quantize).  K % (4*block) == 0, K <= 131072. */
+int scmx_quantize_sc(const void* w, int w_is_bf16, int64_t N, int K, int block, uint32_t* codes, uint8_t* bcodes,
+                     float* wscale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

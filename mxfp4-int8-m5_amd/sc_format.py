@@ -96,3 +96,30 @@ def from_mxfp4(nibbles, e8m0):
     if int(status.item()):
         raise ValueError("a row's block exponents span more than 3: not INT8-embeddable")
     return nibbles.contiguous().view(torch.int32).reshape(-1), bc, ws
+
+
+def quantize(w, fmt=None, with_q=True):
+    """(N, K) float weights (torch tensor on the GPU, float32 or bfloat16; a numpy array is uploaded as float32) ->
+    (codes, bcodes, wscale, q) with the SC-MXFP4 quantizer running on the device, bit-identical to the host
+    procedure of the reference (e2e/sc_format.py:105-111, sim/make_testcase.py:26-44).  fmt: DEFAULT (32-blocks) or
+    the 16-block power-of-two format.  q is the INT8 operand [N, K] (None when with_q is false)."""
+    fmt = fmt or DEFAULT
+    if tuple(fmt.mult) != (1, 2, 4, 8) or fmt.bc_bits != 2 or fmt.block not in (16, 32) or \
+            tuple(fmt.code_mag) != tuple(DEFAULT.code_mag):
+        raise ValueError("the device quantizer produces the power-of-two formats with 16- or 32-wide blocks")
+    if isinstance(w, np.ndarray):
+        w = torch.from_numpy(np.ascontiguousarray(w, np.float32)).cuda()
+    if w.dtype not in (torch.float32, torch.bfloat16):
+        w = w.float()
+    w = w.contiguous()
+    n, k = w.shape
+    codes = torch.empty(n * k // 8, dtype=torch.int32, device=w.device)
+    bc = torch.empty((n, k // (4 * fmt.block)), dtype=torch.uint8, device=w.device)
+    ws = torch.empty(n, dtype=torch.float32, device=w.device)
+    _lib.call("scmx_quantize_sc", _lib.ptr(w), int(w.dtype == torch.bfloat16), n, k, fmt.block, _lib.ptr(codes),
+              _lib.ptr(bc), _lib.ptr(ws), _lib.stream())
+    q = None
+    if with_q:
+        q = torch.empty((n, k), dtype=torch.int8, device=w.device)
+        _lib.call("scmx_unpack_i8", fmt.c_struct(), _lib.ptr(codes), _lib.ptr(bc), _lib.ptr(q), n, k, _lib.stream())
+    return codes, bc, ws, q
