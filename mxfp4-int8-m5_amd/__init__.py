@@ -5,7 +5,8 @@ Modules keep the names of the reference's kernel call surface so model code can 
     sc_kernels  dense prefill kernels (unpack_i8, act_quant, mm_epi, rmsnorm_quant, ...)
     sc_moe      route_sort, moe_mm, moe_combine
     sc_decode   gemv
+    sc_weights  PackedWeight, safetensors caches of packed weights, standard-MXFP4 scale export
 All compute runs in libscmx.so (hand-written HIP for gfx950); importing the kernels without it raises."""
-from . import _lib, sc_format, sc_kernels, sc_moe, sc_decode  # noqa: F401
+from . import _lib, sc_format, sc_kernels, sc_moe, sc_decode, sc_weights  # noqa: F401
 
-__all__ = ["sc_format", "sc_kernels", "sc_moe", "sc_decode"]
+__all__ = ["sc_format", "sc_kernels", "sc_moe", "sc_decode", "sc_weights"]

@@ -104,3 +104,34 @@ def test_rejects_bad_arguments(SF):
         SF.quantize(w)            # K not a multiple of 4 blocks
     with pytest.raises(ValueError):
         SF.quantize(torch.zeros((4, 128), device="cuda"), product_format(layout.Format(block=32, mult=(1, 2, 3, 4))))
+
+
+def test_pack_save_load_and_run(SF, tmp_path):
+    """pack_weights (device quantizer) -> safetensors cache -> PackedWeight (q|k|v rows concatenated) -> GEMM: the
+    result equals the oracle's linear layer on the oracle-quantized weights, bit for bit."""
+    from mxfp4_int8_m5_amd import sc_kernels as S, sc_weights as W
+    from oracle import linear
+    rng = np.random.default_rng(9)
+    k, m = 512, 80
+    ws = {f"layers.0.{p}": torch.from_numpy(llm_weights(rng, n, k).astype(F32)) for p, n in
+          zip(W.GROUPS["qkv"], (128, 64, 64))}
+    ws["layers.0.experts.up_proj"] = torch.from_numpy(llm_weights(rng, 2 * 64, k).astype(F32).reshape(2, 64, k))
+    path = str(tmp_path / "packed.safetensors")
+    W.save_cache(path, W.pack_weights(ws))
+    cache = W.load_cache(path)
+    assert "layers.0.experts.up_proj.1" in cache
+    for key, w in ws.items():                     # the cache holds exactly the oracle's quantization
+        mats = {key: w} if w.dim() == 2 else {f"{key}.{e}": w[e] for e in range(w.shape[0])}
+        for k2, mat in mats.items():
+            c, b, s, _ = layout.quantize(mat.numpy().astype(np.float64))
+            assert all(np.array_equal(x, y) for x, y in zip(cache[k2], (c, b, s)))
+    pw = W.PackedWeight([cache[f"layers.0.{p}"] for p in W.GROUPS["qkv"]])
+    assert pw.splits == [128, 64, 64]
+    xb = bf16.to_bits(rng.standard_normal((m, k)).astype(F32))
+    x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    xq, xs = S.act_quant(x, m)
+    y = host(S.mm_epi(xq, pw.unpack(), xs, pw.wscale, 1))
+    q = np.concatenate([layout.decode(*cache[f"layers.0.{p}"][:2], n, k) for p, n in zip(W.GROUPS["qkv"], (128, 64, 64))])
+    oq, os_ = linear.act_quant(bf16.from_bits(xb))
+    want = linear.epilogue(linear.int_gemm(oq, q), os_, host(pw.wscale), 1)
+    assert np.array_equal(y[:m], want)
