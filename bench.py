@@ -87,6 +87,7 @@ def main():
     ap.add_argument("--no-moe", action="store_true", help="skip the grouped mixture-of-experts leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 512 / 8192 prefill sweep")
     ap.add_argument("--no-quant", action="store_true", help="skip the device quantizer leg")
+    ap.add_argument("--no-model", action="store_true", help="skip the whole-model prefill / decode leg")
     ap.add_argument("--profile-copy", action="store_true",
                     help="first run one plain 256 MiB device copy: the known-size kernel that calibrates FETCH_SIZE / "
                          "WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -328,6 +329,63 @@ def main():
             quant["cpu_oracle_gweights_per_s"] = round(256 * k / (time.perf_counter() - t0) / 1e9, 4)
         del wf, qc, qb, qw
 
+    # ---- whole model: Qwen3-1.7B architecture with random packed weights, prefill and batch-1 decode -----------------
+    model = {}
+    if not a.no_model:
+        torch.cuda.empty_cache()
+        from mxfp4_int8_m5_amd import fused_qwen3 as FQ
+        args = FQ.Qwen3Args()                          # 28 layers, hidden 2048, intermediate 6144, 16 / 8 heads of 128
+        g = torch.Generator(device=dev).manual_seed(0)
+        D, Fi, hq, hk, d = (args.hidden_size, args.intermediate_size, args.num_attention_heads,
+                            args.num_key_value_heads, args.head_dim)
+        shapes = {"self_attn.q_proj": (hq * d, D), "self_attn.k_proj": (hk * d, D), "self_attn.v_proj": (hk * d, D),
+                  "self_attn.o_proj": (D, hq * d), "mlp.gate_proj": (Fi, D), "mlp.up_proj": (Fi, D),
+                  "mlp.down_proj": (D, Fi)}
+
+        def rand_packed(n, k):                         # random codes; shifts 0..3; row scales near 2^-7 / sqrt(k / 2048)
+            codes = torch.randint(-2 ** 31, 2 ** 31 - 1, (n * k // 8,), dtype=torch.int32, device=dev, generator=g)
+            bc = torch.randint(0, 256, (n, k // 128), dtype=torch.uint8, device=dev, generator=g)
+            return codes, bc, torch.full((n,), 2.0 ** -10 * (2048 / k) ** 0.5, device=dev)
+        ones = lambda n: torch.ones(n, dtype=torch.bfloat16, device=dev)   # noqa: E731
+        params = {"model.embed_tokens.weight": (torch.randn((args.vocab_size, D), device=dev, generator=g) * 0.05),
+                  "model.norm.weight": ones(D)}
+        packed = {}
+        for i in range(args.num_hidden_layers):
+            pre = f"model.layers.{i}."
+            params.update({pre + "input_layernorm.weight": ones(D), pre + "post_attention_layernorm.weight": ones(D),
+                           pre + "self_attn.q_norm.weight": ones(d), pre + "self_attn.k_norm.weight": ones(d)})
+            for n, (o, k) in shapes.items():
+                packed[f"layers.{i}.{n}"] = rand_packed(o, k)
+        fm = FQ.FusedQwen3(args, params, packed)
+        del params, packed
+        ids = torch.randint(0, args.vocab_size, (M_TOKENS,), device=dev, generator=g)
+        fm.hidden(ids)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(3):
+            fm.hidden(ids)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms_p = e0.elapsed_time(e1) / 3
+        model = {"workload": "Qwen3-1.7B architecture (28 blocks), random packed weights; prefill of 2048 tokens into "
+                             "a fresh cache (hidden states), then batch-1 decode steps with the bf16 output head",
+                 "prefill_ms": round(ms_p, 2), "prefill_tokens_per_s": round(M_TOKENS / ms_p * 1e3, 0)}
+        for name, kw in (("decode_eager", {}), ("decode_graph_per_half_block", {"graphs": True}),
+                         ("decode_graph_per_step", {"graphs": "step"})):
+            cache = fm.make_cache(512)
+            fm.hidden(ids[:128], cache)
+            dec = FQ.DecodeQwen3(fm, **kw)
+            for j in range(3):
+                dec.step(ids[128 + j:129 + j], cache)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for j in range(32):
+                dec.step(ids[131 + j:132 + j], cache)
+            torch.cuda.synchronize()
+            model[name + "_tokens_per_s"] = round(32 / (time.perf_counter() - t0), 1)
+        del fm, dec, cache
+        torch.cuda.empty_cache()
+
     result = {
         "metric": "INT8 TOPS, W4A8 prefill GEMM M=2048 (Qwen3-1.7B layer shapes), 1 GPU; decode GEMV GB/s alongside",
         "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -342,6 +400,7 @@ def main():
         "moe": moe,
         "decode": decode,
         "quantize": quant,
+        "model": model,
     }
     if not a.no_cpu:
         result["cpu_baseline"] = cpu_baseline()

@@ -69,8 +69,11 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     const int num_n = (a.N + BN - 1) / BN;
     int m0, n0, row_end, expert = 0;
     if (a.tstart) {   // grouped: row tiles of BM inside expert segments
-        const int slot = blockIdx.x / num_n;
-        n0 = (blockIdx.x % num_n) * BN;
+        // Workgroup b runs on XCD b % 8: inside every chunk of 8 row tiles each XCD takes one row tile with all of
+        // its column tiles, so an activation panel is fetched into one L2 only.
+        const int j = blockIdx.x % (8 * num_n);
+        const int slot = blockIdx.x / (8 * num_n) * 8 + (j & 7);
+        n0 = (j >> 3) * BN;
         const int E = a.n_experts;
         if (slot >= a.tstart[E]) return;
         int lo = 0, hi = E;   // largest e with tstart[e] <= slot
@@ -86,8 +89,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         int pid = blockIdx.x;
         const int total = num_m * num_n;
         if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);   // neighbours in tile order share an XCD
-        n0 = (pid / num_m) * BN;
-        m0 = (pid % num_m) * BM;
+        // Tile order: bands of 4 row tiles, inside a band column by column.  The 32 workgroups an XCD runs at once
+        // then share 4 activation panels and 8 weight panels (what its L2 holds) however large M is.
+        constexpr int GM = 4;
+        const int band = pid / (GM * num_n), r = pid % (GM * num_n);
+        const int rows_in_band = min(GM, num_m - band * GM);
+        n0 = (r / rows_in_band) * BN;
+        m0 = (band * GM + r % rows_in_band) * BM;
         row_end = a.M;
     }
     const int K = a.K;
@@ -469,6 +477,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
 template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2>
 static void launch_tile(const GemmArgs& a, int bmode, int row_tiles, hipStream_t s) {
     const int num_n = (a.N + BN - 1) / BN;
+    if (a.tstart) row_tiles = (row_tiles + 7) & ~7;   // grouped: whole chunks of 8 row-tile slots (spare slots exit at once)
     const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * 64);
     if (bmode == B_INT8)
         gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD><<<grid, block, 0, s>>>(a);

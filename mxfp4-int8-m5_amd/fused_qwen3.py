@@ -1,0 +1,333 @@
+"""Qwen3 (dense) prefill and batch-1 decode driven through the W4A8 kernels: the torch-ROCm counterpart of the
+reference's model integrations e2e/fused_qwen3.py:82-301 (FusedQwen3) and e2e/decode.py:29-99 (DecodeQwen3).
+
+Every linear of a block runs as SC-MXFP4 W4A8 (per-token INT8 activations, exact integer accumulation, scaling /
+residual / SwiGLU epilogues); RoPE, the KV cache and attention are plain torch ops, as they are MLX ops in the
+reference.  Weights arrive in Hugging Face layout: a dict of the non-linear parameters plus the packed linears under
+the reference's cache keys "layers.{i}.{path}" (sc_weights.load_cache / pack_weights).
+
+epilogue="gemm": scales, residual adds and SwiGLU in the GEMM's registers (bf16 out), e2e/fused_qwen3.py:224-255.
+epilogue="row":  INT32 GEMM out, then the row kernels res_norm_quant / swiglu_quant / qkv_epilogue_headnorm,
+                 e2e/fused_qwen3.py:257-308.
+The decode step's fixed-shape halves can be captured in HIP graphs (graphs=True), which is what mx.compile does for
+the reference (e2e/decode.py:30-33): one graph launch replaces about ten kernel launches per layer."""
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as TF
+
+from . import sc_decode as G
+from . import sc_format as F
+from . import sc_kernels as S
+from .sc_weights import GROUPS, PackedWeight, pack_weights
+
+BF = torch.bfloat16
+
+
+@dataclass
+class Qwen3Args:
+    hidden_size: int = 2048
+    intermediate_size: int = 6144
+    num_hidden_layers: int = 28
+    num_attention_heads: int = 16
+    num_key_value_heads: int = 8
+    head_dim: int = 128
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1e6
+    vocab_size: int = 151936
+    tie_word_embeddings: bool = True
+
+
+class KVCache:
+    """Per-layer keys / values [heads, max_len, d] with a write offset (mlx_lm's KVCache.update_and_fetch)."""
+
+    def __init__(self, args, max_len, device="cuda"):
+        shape = (args.num_key_value_heads, max_len, args.head_dim)
+        self.k = torch.zeros(shape, dtype=BF, device=device)
+        self.v = torch.zeros(shape, dtype=BF, device=device)
+        self.offset = 0
+
+    def update_and_fetch(self, k, v):
+        n = k.shape[1]
+        if self.offset + n > self.k.shape[1]:
+            raise ValueError("KV cache is full")
+        self.k[:, self.offset:self.offset + n] = k
+        self.v[:, self.offset:self.offset + n] = v
+        self.offset += n
+        return self.k[:, :self.offset], self.v[:, :self.offset]
+
+
+def rms_norm(x, w, eps):
+    v = x.float()
+    return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+
+
+class FusedQwen3:
+    def __init__(self, args, params, packed, resident=False, epilogue="gemm", fmt=None, device="cuda"):
+        """params: "model.embed_tokens.weight", "model.norm.weight", per layer "model.layers.{i}.input_layernorm.weight",
+        ".post_attention_layernorm.weight", ".self_attn.q_norm.weight", ".self_attn.k_norm.weight" (+ "lm_head.weight"
+        when the embeddings are not tied).  packed: {"layers.{i}.{path}": (codes, bcodes, wscale)}."""
+        assert epilogue in ("gemm", "row")
+        self.args, self.epilogue, self.device = args, epilogue, device
+        self.fmt = fmt if fmt is not None else F.Format()
+        self.eps = float(args.rms_norm_eps)
+        dev = lambda k: params[k].to(device=device, dtype=BF).contiguous()   # noqa: E731
+        self.embed = dev("model.embed_tokens.weight")
+        self.norm = dev("model.norm.weight")
+        self.lm_head = self.embed if args.tie_word_embeddings else dev("lm_head.weight")
+        perm = {"gu": S.interleave_gate_up(args.intermediate_size)} if epilogue == "gemm" else {}
+        self.layers = []
+        for i in range(args.num_hidden_layers):
+            p = f"model.layers.{i}."
+            norms = {n: dev(p + n + ".weight") for n in
+                     ("input_layernorm", "post_attention_layernorm", "self_attn.q_norm", "self_attn.k_norm")}
+            ws = {g: PackedWeight([packed[f"layers.{i}.{path}"] for path in paths], resident, perm.get(g), self.fmt,
+                                  device) for g, paths in GROUPS.items()}
+            self.layers.append((norms, ws))
+        half = args.head_dim // 2
+        self.inv_freq = 1.0 / (args.rope_theta ** (torch.arange(half, device=device, dtype=torch.float32) / half))
+
+    @classmethod
+    def from_float(cls, args, state, **kw):
+        """state: Hugging Face state dict with the block linears as float tensors; they are quantized on the GPU."""
+        lin = {f"layers.{i}.{path}": state[f"model.layers.{i}.{path}.weight"]
+               for i in range(args.num_hidden_layers) for paths in GROUPS.values() for path in paths}
+        flat = pack_weights(lin, kw.get("fmt"))
+        packed = {k: (flat[k + ".codes"], flat[k + ".bcodes"], flat[k + ".wscale"]) for k in lin}
+        return cls(args, state, packed, **kw)
+
+    def weight_bytes(self):
+        return sum(w.nbytes() for _, ws in self.layers for w in ws.values())
+
+    def make_cache(self, max_len=4096):
+        return [KVCache(self.args, max_len, self.device) for _ in self.layers]
+
+    # ---- pieces shared by prefill and decode --------------------------------------------------------------------
+    def rope(self, x, offset):
+        """x [heads, L, d]: rotation of the (i, i + d/2) pairs at positions offset .. offset+L-1 (mlx nn.RoPE,
+        traditional=False)."""
+        L = x.shape[1]
+        ang = (torch.arange(offset, offset + L, device=x.device, dtype=torch.float32))[:, None] * self.inv_freq[None]
+        cos, sin = ang.cos()[None], ang.sin()[None]
+        x1, x2 = x.float().chunk(2, -1)
+        return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], -1).to(x.dtype)
+
+    def _attention(self, c, q, k, v, L):
+        """q [hq, L, d], k / v [hk, L, d] of the new positions -> [L, hq * d]."""
+        off = c.offset
+        q, k = self.rope(q, off), self.rope(k, off)
+        k, v = c.update_and_fetch(k, v)
+        rep = q.shape[0] // k.shape[0]
+        if rep > 1:
+            k, v = k.repeat_interleave(rep, 0), v.repeat_interleave(rep, 0)
+        if L == 1:
+            o = TF.scaled_dot_product_attention(q[None], k[None], v[None])
+        elif off == 0:
+            o = TF.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)
+        else:
+            pos = torch.arange(off, off + L, device=q.device)[:, None]
+            mask = torch.arange(off + L, device=q.device)[None] <= pos
+            o = TF.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask)
+        return o[0].transpose(0, 1).reshape(L, -1).contiguous()
+
+    def _embed(self, ids):
+        h = self.embed[ids.reshape(-1)]
+        L = h.shape[0]
+        Mp = S.pad_rows(L)
+        if Mp != L:
+            h = TF.pad(h, (0, 0, 0, Mp - L))
+        return h.contiguous(), L, Mp
+
+    # ---- prefill ------------------------------------------------------------------------------------------------
+    def hidden(self, ids, cache=None):
+        """Final normed hidden states [L, D] for prompt ids [L] (prefill into a fresh or offset cache)."""
+        S.set_format(self.fmt)
+        cache = cache if cache is not None else self.make_cache(max(4096, ids.numel()))
+        return (self._hidden_gemm_epi if self.epilogue == "gemm" else self._hidden_row_epi)(ids, cache)
+
+    def _hidden_gemm_epi(self, ids, cache):
+        a = self.args
+        hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
+        h, L, Mp = self._embed(ids)
+        nl = len(self.layers)
+        xq, xs = S.rmsnorm_quant(h, self.layers[0][0]["input_layernorm"], self.eps, Mp)
+        for i, (nw, ws) in enumerate(self.layers):
+            y = S.mm_epi(xq, ws["qkv"].unpack(), xs, ws["qkv"].wscale, 1)
+            q, k, v = S.qkv_headnorm_y(y, nw["self_attn.q_norm"], nw["self_attn.k_norm"], self.eps, L, hq, hk, d)
+            o = self._attention(cache[i], q, k, v, L)
+            xq, xs = S.act_quant(o, Mp)
+            h = S.mm_epi(xq, ws["o"].unpack(), xs, ws["o"].wscale, 2, res=h)
+            xq, xs = S.rmsnorm_quant(h, nw["post_attention_layernorm"], self.eps)
+            act = S.mm_epi(xq, ws["gu"].unpack(), xs, ws["gu"].wscale, 3)
+            xq, xs = S.act_quant(act, nt=512)
+            h = S.mm_epi(xq, ws["down"].unpack(), xs, ws["down"].wscale, 2, res=h)
+            if i + 1 < nl:
+                xq, xs = S.rmsnorm_quant(h, self.layers[i + 1][0]["input_layernorm"], self.eps)
+        return rms_norm(h[:L], self.norm, self.eps)
+
+    def _hidden_row_epi(self, ids, cache):
+        a = self.args
+        hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
+        h, L, Mp = self._embed(ids)
+        nl = len(self.layers)
+        xq, xs = S.rmsnorm_quant(h, self.layers[0][0]["input_layernorm"], self.eps, Mp)
+        for i, (nw, ws) in enumerate(self.layers):
+            acc = S.mm_i8_i32(xq, ws["qkv"].unpack())
+            q, k, v = S.qkv_epilogue_headnorm(acc, xs, ws["qkv"].wscale, nw["self_attn.q_norm"], nw["self_attn.k_norm"],
+                                              self.eps, L, hq, hk, d)
+            o = self._attention(cache[i], q, k, v, L)
+            xq, xs = S.act_quant(o, Mp)
+            acc = S.mm_i8_i32(xq, ws["o"].unpack())
+            h, xq, xs = S.res_norm_quant(acc, xs, ws["o"].wscale, h, nw["post_attention_layernorm"], self.eps)
+            acc = S.mm_i8_i32(xq, ws["gu"].unpack())
+            xq, xs = S.swiglu_quant(acc, xs, ws["gu"].wscale)
+            acc = S.mm_i8_i32(xq, ws["down"].unpack())
+            if i + 1 < nl:
+                h, xq, xs = S.res_norm_quant(acc, xs, ws["down"].wscale, h, self.layers[i + 1][0]["input_layernorm"],
+                                             self.eps)
+            else:
+                h = S.res_epilogue(acc, xs, ws["down"].wscale, h)
+        return rms_norm(h[:L], self.norm, self.eps)
+
+    def logits(self, h):
+        return h @ self.lm_head.T
+
+    def __call__(self, ids, cache=None):
+        """Logits for every position."""
+        return self.logits(self.hidden(ids, cache))
+
+
+class DecodeQwen3:
+    """Batch-1 decode from a FusedQwen3 with epilogue="gemm": W4A8 GEMVs on the packed weights
+    (e2e/decode.py:29-99).  fuse_prologue="act" (default): RMSNorm + INT8 as separate kernels, the per-token INT8 of
+    the o / down inputs inside those GEMVs' prologues; True: every quantization in a GEMV prologue; False: all
+    separate.  graphs=True captures the two fixed-shape halves of every layer in HIP graphs on first use;
+    graphs="step" captures the whole step (all layers, attention over the full cache buffer under a position mask,
+    output head) as one graph per cache."""
+
+    def __init__(self, fused, fuse_prologue="act", graphs=False, head=True):
+        assert fused.epilogue == "gemm"
+        self.f, self.args, self.fuse, self.head = fused, fused.args, fuse_prologue, head
+        self.graphs = {} if graphs else None
+        self.whole_step = graphs == "step"
+
+    def _pre(self, h, nw, w):
+        f, a = self.f, self.args
+        hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
+        if self.fuse is True:
+            y = G.gemv(h, w.codes, w.bcodes, None, w.wscale, w.N, 1, pro=2, nw=nw["input_layernorm"], eps=f.eps,
+                       fmt=f.fmt)
+        else:
+            xq, xs = S.rmsnorm_quant(h, nw["input_layernorm"], f.eps, 1)
+            y = G.gemv(xq, w.codes, w.bcodes, xs, w.wscale, w.N, 1, fmt=f.fmt)
+        return S.qkv_headnorm_y(y[None], nw["self_attn.q_norm"], nw["self_attn.k_norm"], f.eps, 1, hq, hk, d)
+
+    def _post(self, o, h, nw, ws):
+        f = self.f
+        wo, wg, wd = ws["o"], ws["gu"], ws["down"]
+        if self.fuse:
+            h = G.gemv(o, wo.codes, wo.bcodes, None, wo.wscale, wo.N, 2, res=h, pro=1, fmt=f.fmt)[None]
+        else:
+            xq, xs = S.act_quant(o, 1)
+            h = G.gemv(xq, wo.codes, wo.bcodes, xs, wo.wscale, wo.N, 2, res=h, fmt=f.fmt)[None]
+        if self.fuse is True:
+            act = G.gemv(h, wg.codes, wg.bcodes, None, wg.wscale, wg.N, 3, pro=2, nw=nw["post_attention_layernorm"],
+                         eps=f.eps, fmt=f.fmt)
+        else:
+            xq, xs = S.rmsnorm_quant(h, nw["post_attention_layernorm"], f.eps, 1)
+            act = G.gemv(xq, wg.codes, wg.bcodes, xs, wg.wscale, wg.N, 3, fmt=f.fmt)
+        if self.fuse:
+            return G.gemv(act[None], wd.codes, wd.bcodes, None, wd.wscale, wd.N, 2, res=h, pro=1, fmt=f.fmt)[None]
+        xq, xs = S.act_quant(act[None], 1)
+        return G.gemv(xq, wd.codes, wd.bcodes, xs, wd.wscale, wd.N, 2, res=h, fmt=f.fmt)[None]
+
+    def _graphed(self, key, fn, inputs):
+        """Capture fn(*static inputs) once per key; later calls copy the inputs in and replay."""
+        if key not in self.graphs:
+            static = [t.clone() for t in inputs]
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                fn(*static)                                   # warm-up outside the capture
+            torch.cuda.current_stream().wait_stream(s)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                out = fn(*static)
+            self.graphs[key] = (g, static, out)
+        g, static, out = self.graphs[key]
+        for dst, src in zip(static, inputs):
+            dst.copy_(src)
+        g.replay()
+        return out
+
+    # ---- the whole step as one HIP graph -----------------------------------------------------------------------
+    # Everything that changes from token to token lives in device memory (token id, position), the KV cache is
+    # written with an index copy at the position and attention runs over the whole cache buffer under a position
+    # mask, so the launch sequence is identical for every token and one graph replay per token replaces
+    # ~25 launches and their host-side preparation per layer.
+    def _step_static(self, tok, pos, cache):
+        f, a = self.f, self.args
+        hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
+        h = f.embed.index_select(0, tok)
+        ang = pos.to(torch.float32)[:, None] * f.inv_freq[None]
+        cos, sin = ang.cos()[None], ang.sin()[None]
+
+        def rope(x):
+            x1, x2 = x.float().chunk(2, -1)
+            return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], -1).to(x.dtype)
+        mask = (torch.arange(cache[0].k.shape[1], device=tok.device)[None] <= pos[:, None])[None, None]
+        for i, (nw, ws) in enumerate(f.layers):
+            q, k, v = self._pre(h, nw, ws["qkv"])
+            c = cache[i]
+            c.k.index_copy_(1, pos, rope(k))
+            c.v.index_copy_(1, pos, v)
+            # the hq / hk query heads that share a KV head take the place of the (length-1) query sequence
+            o = TF.scaled_dot_product_attention(rope(q).view(1, hk, hq // hk, d), c.k[None], c.v[None], attn_mask=mask)
+            h = self._post(o.reshape(1, hq * d), h, nw, ws)
+        hn = rms_norm(h, f.norm, f.eps)
+        return f.logits(hn) if self.head else hn
+
+    def _step_graph(self, tok, cache):
+        key = ("step", id(cache))
+        if key not in self.graphs:
+            st_tok = tok.reshape(-1)[:1].clone()
+            st_pos = torch.zeros(1, dtype=torch.int64, device=tok.device)
+            st_pos.fill_(cache[0].offset)
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                self._step_static(st_tok, st_pos, cache)      # warm-up outside the capture (writes this token's row)
+            torch.cuda.current_stream().wait_stream(s)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                out = self._step_static(st_tok, st_pos, cache)
+            self.graphs[key] = (g, st_tok, st_pos, out, cache)
+        g, st_tok, st_pos, out, _ = self.graphs[key]
+        if cache[0].offset >= cache[0].k.shape[1]:
+            raise ValueError("KV cache is full")
+        st_tok.copy_(tok.reshape(-1)[:1])
+        st_pos.fill_(cache[0].offset)
+        g.replay()
+        for c in cache:
+            c.offset += 1
+        return out
+
+    def step(self, tok, cache):
+        """tok: int64 [1] -> logits [1, V] (or the final hidden row when head is False)."""
+        f = self.f
+        S.set_format(f.fmt)
+        if self.whole_step:
+            return self._step_graph(tok, cache)
+        h = f.embed[tok.reshape(-1)[:1]].contiguous()   # [1, D]
+        for i, (nw, ws) in enumerate(f.layers):
+            if self.graphs is None:
+                q, k, v = self._pre(h, nw, ws["qkv"])
+            else:
+                q, k, v = self._graphed(("pre", i), lambda x, nw=nw, w=ws["qkv"]: self._pre(x, nw, w), [h])
+            o = f._attention(cache[i], q, k, v, 1)
+            if self.graphs is None:
+                h = self._post(o, h, nw, ws)
+            else:
+                h = self._graphed(("post", i), lambda x, r, nw=nw, ws=ws: self._post(x, r, nw, ws), [o, h])
+        hn = rms_norm(h, f.norm, f.eps)
+        return f.logits(hn) if self.head else hn

@@ -1,0 +1,162 @@
+"""Model-level checks of the Qwen3 integration (prefill in both epilogue styles, batch-1 decode, HIP-graph replay)
+on a small random model.  The kernels themselves are pinned bit-exactly elsewhere; here the composition is checked
+against a plain float32 torch model that uses the dequantized weights, within the W4A8 tolerance, and the decode path
+against the prefill path, as the reference does in e2e/check_fused.py and e2e/check_decode.py."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tiny():
+    from mxfp4_int8_m5_amd import fused_qwen3 as Q, sc_weights as W
+    args = Q.Qwen3Args(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                       num_key_value_heads=2, head_dim=64, vocab_size=320, rope_theta=1e4)
+    g = torch.Generator().manual_seed(0)
+    rnd = lambda *s, sc=1.0: torch.randn(*s, generator=g) * sc   # noqa: E731
+    state = {"model.embed_tokens.weight": rnd(args.vocab_size, args.hidden_size),
+             "model.norm.weight": 1 + rnd(args.hidden_size, sc=0.1)}
+    shapes = {"self_attn.q_proj": (256, 256), "self_attn.k_proj": (128, 256), "self_attn.v_proj": (128, 256),
+              "self_attn.o_proj": (256, 256), "mlp.gate_proj": (512, 256), "mlp.up_proj": (512, 256),
+              "mlp.down_proj": (256, 512)}
+    for i in range(args.num_hidden_layers):
+        p = f"model.layers.{i}."
+        for n in ("input_layernorm", "post_attention_layernorm"):
+            state[p + n + ".weight"] = 1 + rnd(args.hidden_size, sc=0.1)
+        for n in ("self_attn.q_norm", "self_attn.k_norm"):
+            state[p + n + ".weight"] = 1 + rnd(args.head_dim, sc=0.1)
+        for n, (o, k) in shapes.items():
+            state[p + n + ".weight"] = rnd(o, k, sc=k ** -0.5)
+    state = {k: v.to(torch.bfloat16).float() for k, v in state.items()}     # bf16-representable parameters
+    lin = {f"layers.{i}.{n}": state[f"model.layers.{i}.{n}.weight"] for i in range(2) for n in shapes}
+    flat = W.pack_weights(lin)
+    packed = {k: (flat[k + ".codes"], flat[k + ".bcodes"], flat[k + ".wscale"]) for k in lin}
+    return Q, args, state, packed
+
+
+def float_model(Q, args, state, packed, ids):
+    """float32 torch on the CPU: the same network with the dequantized 4-bit weights and no activation quantization."""
+    from oracle import layout
+    a = args
+    hq, hk, d, eps = a.num_attention_heads, a.num_key_value_heads, a.head_dim, a.rms_norm_eps
+
+    def weight(i, n):
+        c, b, s = packed[f"layers.{i}.{n}"]
+        rows = s.shape[0]
+        k = c.size * 8 // rows
+        return torch.from_numpy(layout.decode(c, b, rows, k).astype(np.float32) * s[:, None])
+
+    def norm(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+
+    def rope(x):
+        L = x.shape[1]
+        half = d // 2
+        inv = 1.0 / (a.rope_theta ** (torch.arange(half, dtype=torch.float32) / half))
+        ang = torch.arange(L, dtype=torch.float32)[:, None] * inv[None]
+        x1, x2 = x.chunk(2, -1)
+        return torch.cat([x1 * ang.cos() - x2 * ang.sin(), x2 * ang.cos() + x1 * ang.sin()], -1)
+
+    h = state["model.embed_tokens.weight"][ids]
+    L = h.shape[0]
+    for i in range(a.num_hidden_layers):
+        p = f"model.layers.{i}."
+        x = norm(h, state[p + "input_layernorm.weight"])
+        q = (x @ weight(i, "self_attn.q_proj").T).view(L, hq, d).transpose(0, 1)
+        k = (x @ weight(i, "self_attn.k_proj").T).view(L, hk, d).transpose(0, 1)
+        v = (x @ weight(i, "self_attn.v_proj").T).view(L, hk, d).transpose(0, 1)
+        q, k = rope(norm(q, state[p + "self_attn.q_norm.weight"])), rope(norm(k, state[p + "self_attn.k_norm.weight"]))
+        k, v = k.repeat_interleave(hq // hk, 0), v.repeat_interleave(hq // hk, 0)
+        o = torch.nn.functional.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+        h = h + o.transpose(0, 1).reshape(L, -1) @ weight(i, "self_attn.o_proj").T
+        x = norm(h, state[p + "post_attention_layernorm.weight"])
+        g, u = x @ weight(i, "mlp.gate_proj").T, x @ weight(i, "mlp.up_proj").T
+        h = h + (torch.nn.functional.silu(g) * u) @ weight(i, "mlp.down_proj").T
+    return norm(h, state["model.norm.weight"])
+
+
+def rel(a, b):
+    a, b = a.float().cpu(), b.float().cpu()
+    return float((a - b).norm() / b.norm())
+
+
+@pytest.mark.parametrize("epilogue", ["gemm", "row"])
+def test_prefill_against_float_model(tiny, epilogue):
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (70,), generator=torch.Generator().manual_seed(1))
+    m = Q.FusedQwen3(args, state, packed, epilogue=epilogue)
+    h = m.hidden(ids.cuda())
+    ref = float_model(Q, args, state, packed, ids)
+    assert h.shape == ref.shape
+    assert rel(h, ref) < 3e-2, rel(h, ref)       # two blocks of INT8 activations + bf16 residual stream
+
+
+def test_resident_int8_weights_give_the_same_result(tiny):
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (33,), generator=torch.Generator().manual_seed(2)).cuda()
+    a = Q.FusedQwen3(args, state, packed).hidden(ids)
+    b = Q.FusedQwen3(args, state, packed, resident=True).hidden(ids)
+    assert torch.equal(a, b)                       # fused unpack and the INT8 copy feed the same integers to the MFMAs
+
+
+def test_from_float_quantizes_on_the_device(tiny):
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (20,), generator=torch.Generator().manual_seed(3)).cuda()
+    a = Q.FusedQwen3(args, state, packed).hidden(ids)
+    b = Q.FusedQwen3.from_float(args, state).hidden(ids)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("fuse", ["act", True, False])
+def test_decode_continues_the_prefill(tiny, fuse):
+    """Prefill L tokens, decode the next 3 one by one: the hidden rows equal those of one prefill over L + 3 tokens
+    up to the attention kernels' rounding (the linears see identical INT8 rows in both paths)."""
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (40,), generator=torch.Generator().manual_seed(4)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    full = m.hidden(ids)
+    cache = m.make_cache(64)
+    m.hidden(ids[:37], cache)
+    dec = Q.DecodeQwen3(m, fuse_prologue=fuse, head=False)
+    rows = torch.cat([dec.step(ids[37 + j:38 + j], cache) for j in range(3)])
+    assert cache[0].offset == 40
+    assert rel(rows, full[37:]) < 2e-2, rel(rows, full[37:])
+
+
+def test_decode_graph_replays_match_eager_steps(tiny):
+    """Each captured half is replayed on every step; between replays the program runs its eager attention and cache
+    updates.  Every step's logits must equal the eager decoder's bit for bit."""
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (24,), generator=torch.Generator().manual_seed(5)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    c1, c2 = m.make_cache(64), m.make_cache(64)
+    m.hidden(ids[:16], c1)
+    m.hidden(ids[:16], c2)
+    eager, graphed = Q.DecodeQwen3(m), Q.DecodeQwen3(m, graphs=True)
+    for j in range(16, 24):
+        a = eager.step(ids[j:j + 1], c1)
+        b = graphed.step(ids[j:j + 1], c2)
+        torch.cuda.synchronize()
+        assert a.shape == (1, args.vocab_size) and torch.equal(a, b), j
+
+
+def test_whole_step_graph_follows_the_eager_decoder(tiny):
+    """One graph per step with attention over the whole cache buffer under a position mask: equal to the eager
+    decoder up to the attention kernel's summation order, on every replay (positions and tokens change between
+    replays, and so does the cache content the replayed kernels read)."""
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (30,), generator=torch.Generator().manual_seed(6)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    c1, c2 = m.make_cache(48), m.make_cache(48)
+    m.hidden(ids[:16], c1)
+    m.hidden(ids[:16], c2)
+    eager, graphed = Q.DecodeQwen3(m, head=False), Q.DecodeQwen3(m, graphs="step", head=False)
+    for j in range(16, 30):
+        a = eager.step(ids[j:j + 1], c1)
+        b = graphed.step(ids[j:j + 1], c2).clone()
+        torch.cuda.synchronize()
+        assert c2[0].offset == j + 1
+        assert rel(b, a) < 1e-2, (j, rel(b, a))
+    assert rel(c2[1].k[:, :30], c1[1].k[:, :30]) < 1e-2 and float(c2[1].k[:, 30:].abs().max()) == 0.0
