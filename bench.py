@@ -259,9 +259,11 @@ def main():
         e1.record(stream)
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / reps_m
+        tiles = int(SM.route_sort(inds, E, TM)[4][-1].item())
         ops = 2.0 * R * 3 * Fi * D
         moe = {"workload": "BASELINE configs[3]: act quant + token sort + grouped gate_up GEMM (SwiGLU epilogue) + act "
                            "quant + grouped down GEMM + weighted combine", "tokens": T, "experts": E, "topk": TOPK,
+               "row_tile": TM, "row_tiles": tiles, "padded_rows_pct": round((tiles * TM / R - 1) * 100, 1),
                "ms": round(ms, 4), "tops": round(ops / ms / 1e9, 1),
                "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
         del gu, dn, x
@@ -368,10 +370,14 @@ def main():
         torch.cuda.synchronize()
         ms_p = e0.elapsed_time(e1) / 3
         model = {"workload": "Qwen3-1.7B architecture (28 blocks), random packed weights; prefill of 2048 tokens into "
-                             "a fresh cache (hidden states), then batch-1 decode steps with the bf16 output head",
+                             "a fresh cache (hidden states), then batch-1 decode steps at context 131..163 (bf16 output head unless "
+                             "named otherwise)",
                  "prefill_ms": round(ms_p, 2), "prefill_tokens_per_s": round(M_TOKENS / ms_p * 1e3, 0)}
         for name, kw in (("decode_eager", {}), ("decode_graph_per_half_block", {"graphs": True}),
-                         ("decode_graph_per_step", {"graphs": "step"})):
+                         ("decode_graph_per_step", {"graphs": "step"}),
+                         ("decode_graph_per_step_all_prologues_fused", {"graphs": "step", "fuse_prologue": True}),
+                         ("decode_graph_per_step_all_prologues_fused_packed_head",
+                          {"graphs": "step", "fuse_prologue": True, "head": "packed"})):
             cache = fm.make_cache(512)
             fm.hidden(ids[:128], cache)
             dec = FQ.DecodeQwen3(fm, **kw)

@@ -112,6 +112,25 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
                       const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k, uint16_t* v,
                       int L, int hq, int hk, int d, void* stream);
 
+/* scmx_qkv_headnorm followed by the rotary embedding of q and k (pairs (i, i + d/2) of a head, angle = position *
+ * inv_freq[i], inv_freq f32 [d/2]) and the append to the KV cache: q -> [hq, L, d]; k, v -> rows pos..pos+L-1 of
+ * caches [hk, cache_rows, d].  pos = *pos_dev when pos_dev != NULL (a device-resident position, so that a captured
+ * graph can be replayed for every token), else pos0.  With pos_dev the caller guarantees *pos_dev + L <= cache_rows.
+ * Fuses what the model integrations do with array ops after qkv_headnorm_y: at.rope(q), at.rope(k),
+ * cache.update_and_fetch(k, v) (e2e/fused_qwen3.py:216-221). */
+int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
+                           const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* kcache,
+                           uint16_t* vcache, int L, int hq, int hk, int d, const float* inv_freq,
+                           const int64_t* pos_dev, int64_t pos0, int cache_rows, void* stream);
+
+/* Single-token attention against a KV cache: out bf16 [hq * d] = softmax(q . K^T * scale) V per query head, q bf16
+ * [hq, d], caches bf16 [hk, cache_rows, d] of which the first n rows are valid; n = *pos_dev + 1 when pos_dev != NULL
+ * (device-resident position, for graph replay).  d in {64, 128, 256}.  Takes the place of the
+ * array library's scaled-dot-product attention at L = 1 in the decode step (e2e/decode.py:1-5, e2e/fused_qwen3.py:
+ * 216-222), so that the step is a fixed launch sequence. */
+int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, const int64_t* pos_dev, int n,
+                     uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, void* stream);
+
 /* OLMoE q/k/v split with RMSNorm over the full h*d width.  Replaces qkv_fullnorm_y, e2e/sc_kernels.py:390-423,
  * 629-637. */
 int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q,

@@ -173,14 +173,27 @@ __global__ __launch_bounds__(NT) void swiglu_quant_kernel(const int32_t* __restr
 }
 
 // ---- Qwen3 q/k/v split with per-head RMSNorm: one wave per head, d/64 consecutive values per lane ---------------
+// With inv_freq != NULL the kernel also rotates q and k (pairs (i, i + d/2) of a head, angle = position * inv_freq[i])
+// and writes k and v at rows pos .. pos+L-1 of caches [hk, kv_rows, d] instead of dense [hk, L, d] outputs.
+struct RopeArgs {
+    const float* inv_freq;   // [d / 2] or NULL
+    const int64_t* pos_dev;  // optional device-resident position of row 0 (read when non-NULL), else pos0
+    int64_t pos0;
+    int kv_rows;             // rows per head of the k / v destinations
+};
+
 __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
                                                           const float* __restrict__ wscale, const uint16_t* __restrict__ y,
                                                           const uint16_t* __restrict__ qn, const uint16_t* __restrict__ kn,
                                                           float eps, uint16_t* __restrict__ q, uint16_t* __restrict__ k,
-                                                          uint16_t* __restrict__ v, int L, int hq, int hk, int d) {
+                                                          uint16_t* __restrict__ v, int L, int hq, int hk, int d,
+                                                          const RopeArgs rope) {
     const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int heads = hq + 2 * hk, ntot = heads * d, per = d / 64;
-    for (int g = wave; g < heads; g += NT / 64) {
+    const int64_t pos = rope.inv_freq ? (rope.pos_dev ? rope.pos_dev[0] : rope.pos0) + row : row;
+    const int kv_rows = rope.inv_freq ? rope.kv_rows : L;
+    // blockIdx.y strides over groups of NT / 64 heads (one per wave): a single row still fills many CUs
+    for (int g = blockIdx.y * (NT / 64) + wave; g < heads; g += gridDim.y * (NT / 64)) {
         float yv[8];   // per <= 8 (d <= 512)
         float ss = 0.0f;
         for (int i = 0; i < per; ++i) {
@@ -194,13 +207,25 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
         uint16_t* out;
         int hh;
         if (g < hq) { out = q; hh = g; } else if (g < hq + hk) { out = k; hh = g - hq; } else { out = v; hh = g - hq - hk; }
-        uint16_t* o = out + (size_t(hh) * L + row) * d + per * lane;
+        uint16_t* o = g < hq ? out + (size_t(hh) * L + row) * d + per * lane
+                             : out + (size_t(hh) * kv_rows + size_t(pos)) * d + per * lane;
         if (g < hq + hk) {
             ss = wave_sum(ss);
             const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
             const uint16_t* w = g < hq ? qn : kn;
-            for (int i = 0; i < per; ++i)
-                o[i] = f32_to_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
+            for (int i = 0; i < per; ++i) {
+                float nv = round_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
+                if (rope.inv_freq) {
+                    // element e = per*lane + i pairs with e +- d/2, held by lane +- 32 at the same i
+                    const float other = __shfl_xor(nv, 32, WAVE);
+                    const int e = per * lane + i;
+                    float sn, cs;
+                    sincosf(float(pos) * rope.inv_freq[e % (d / 2)], &sn, &cs);
+                    nv = lane < 32 ? __fsub_rn(__fmul_rn(nv, cs), __fmul_rn(other, sn))
+                                   : __fadd_rn(__fmul_rn(nv, cs), __fmul_rn(other, sn));
+                }
+                o[i] = f32_to_bf16(nv);
+            }
         } else {
             for (int i = 0; i < per; ++i) o[i] = f32_to_bf16(yv[i]);
         }
@@ -461,6 +486,12 @@ int scmx_swiglu_quant(const int32_t* acc, const float* xscale, const float* wsca
     return check_launch("swiglu_quant");
 }
 
+// few rows (decode): spread the heads over workgroups; many rows: one workgroup per row
+static dim3 headnorm_grid(int L, int heads) {
+    const int groups = (heads + NT / 64 - 1) / (NT / 64);
+    return dim3(L, L >= 256 ? 1 : groups);
+}
+
 int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
                       const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k, uint16_t* v, int L,
                       int hq, int hk, int d, void* stream) {
@@ -473,9 +504,32 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
         return SCMX_ERR_ARG;
     }
     if (L == 0) return SCMX_OK;
-    qkv_headnorm_kernel<<<dim3(L), dim3(NT), 0, (hipStream_t)stream>>>(acc, xscale, wscale, y, qn, kn, eps, q, k, v, L, hq,
-                                                                        hk, d);
+    qkv_headnorm_kernel<<<headnorm_grid(L, hq + 2 * hk), dim3(NT), 0, (hipStream_t)stream>>>(
+        acc, xscale, wscale, y, qn, kn, eps, q, k, v, L, hq, hk, d, RopeArgs{nullptr, nullptr, 0, 0});
     return check_launch("qkv_headnorm");
+}
+
+int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
+                           const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* kcache,
+                           uint16_t* vcache, int L, int hq, int hk, int d, const float* inv_freq,
+                           const int64_t* pos_dev, int64_t pos0, int cache_rows, void* stream) {
+    if ((!acc && !y) || (acc && (!xscale || !wscale)) || !qn || !kn || !q || !kcache || !vcache || !inv_freq) {
+        set_error("qkv_headnorm_rope: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (L < 0 || hq < 1 || hk < 1 || d % 64 || d < 64 || d > 512) {
+        set_error("qkv_headnorm_rope: need head dim a multiple of 64 in 64..512 (d=%d)", d);
+        return SCMX_ERR_ARG;
+    }
+    if (cache_rows < L || (!pos_dev && (pos0 < 0 || pos0 + L > cache_rows))) {
+        set_error("qkv_headnorm_rope: rows %lld..%lld do not fit a cache of %d rows", (long long)pos0,
+                  (long long)(pos0 + L), cache_rows);
+        return SCMX_ERR_ARG;
+    }
+    if (L == 0) return SCMX_OK;
+    qkv_headnorm_kernel<<<headnorm_grid(L, hq + 2 * hk), dim3(NT), 0, (hipStream_t)stream>>>(
+        acc, xscale, wscale, y, qn, kn, eps, q, kcache, vcache, L, hq, hk, d, RopeArgs{inv_freq, pos_dev, pos0, cache_rows});
+    return check_launch("qkv_headnorm_rope");
 }
 
 int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k,

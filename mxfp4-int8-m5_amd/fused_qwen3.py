@@ -2,8 +2,9 @@
 reference's model integrations e2e/fused_qwen3.py:82-301 (FusedQwen3) and e2e/decode.py:29-99 (DecodeQwen3).
 
 Every linear of a block runs as SC-MXFP4 W4A8 (per-token INT8 activations, exact integer accumulation, scaling /
-residual / SwiGLU epilogues); RoPE, the KV cache and attention are plain torch ops, as they are MLX ops in the
-reference.  Weights arrive in Hugging Face layout: a dict of the non-linear parameters plus the packed linears under
+residual / SwiGLU epilogues); prefill attention is torch's scaled-dot-product attention (an MLX op in the reference); RoPE and
+the KV-cache append, array ops in the reference, are fused into the q/k/v norm kernel, and the single-token attention
+of the decode step is a kernel of this library that reads the position from device memory.  Weights arrive in Hugging Face layout: a dict of the non-linear parameters plus the packed linears under
 the reference's cache keys "layers.{i}.{path}" (sc_weights.load_cache / pack_weights).
 
 epilogue="gemm": scales, residual adds and SwiGLU in the GEMM's registers (bf16 out), e2e/fused_qwen3.py:224-255.
@@ -103,26 +104,27 @@ class FusedQwen3:
         return [KVCache(self.args, max_len, self.device) for _ in self.layers]
 
     # ---- pieces shared by prefill and decode --------------------------------------------------------------------
-    def rope(self, x, offset):
-        """x [heads, L, d]: rotation of the (i, i + d/2) pairs at positions offset .. offset+L-1 (mlx nn.RoPE,
-        traditional=False)."""
-        L = x.shape[1]
-        ang = (torch.arange(offset, offset + L, device=x.device, dtype=torch.float32))[:, None] * self.inv_freq[None]
-        cos, sin = ang.cos()[None], ang.sin()[None]
-        x1, x2 = x.float().chunk(2, -1)
-        return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], -1).to(x.dtype)
+    def _qkv(self, c, L, nw, y=None, acc=None, xs=None, ws=None, pos=None):
+        """Per-head RMSNorm of q and k, rotary embedding at positions pos..pos+L-1 (pos defaults to the cache offset;
+        an int64 device tensor for graph replay) and the KV-cache append, in one kernel: returns q [hq, L, d]."""
+        a = self.args
+        return S.qkv_headnorm_rope(y, nw["self_attn.q_norm"], nw["self_attn.k_norm"], self.eps, L, a.num_attention_heads,
+                                   a.num_key_value_heads, a.head_dim, c.k, c.v, c.offset if pos is None else pos,
+                                   self.inv_freq, acc=acc, xscale=xs, wscale=ws)
 
-    def _attention(self, c, q, k, v, L):
-        """q [hq, L, d], k / v [hk, L, d] of the new positions -> [L, hq * d]."""
+    def _attend(self, c, q, L):
+        """q [hq, L, d] (already rotated) against the cache, whose rows offset..offset+L-1 were just written."""
         off = c.offset
-        q, k = self.rope(q, off), self.rope(k, off)
-        k, v = c.update_and_fetch(k, v)
-        rep = q.shape[0] // k.shape[0]
-        if rep > 1:
-            k, v = k.repeat_interleave(rep, 0), v.repeat_interleave(rep, 0)
+        if off + L > c.k.shape[1]:
+            raise ValueError("KV cache is full")
+        c.offset = off + L
+        k, v = c.k[:, :off + L], c.v[:, :off + L]
+        hq, hk = q.shape[0], k.shape[0]
         if L == 1:
-            o = TF.scaled_dot_product_attention(q[None], k[None], v[None])
-        elif off == 0:
+            return S.attn_decode(q, c.k, c.v, off + 1)
+        if hq != hk:
+            k, v = k.repeat_interleave(hq // hk, 0), v.repeat_interleave(hq // hk, 0)
+        if off == 0:
             o = TF.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)
         else:
             pos = torch.arange(off, off + L, device=q.device)[:, None]
@@ -153,8 +155,9 @@ class FusedQwen3:
         xq, xs = S.rmsnorm_quant(h, self.layers[0][0]["input_layernorm"], self.eps, Mp)
         for i, (nw, ws) in enumerate(self.layers):
             y = S.mm_epi(xq, ws["qkv"].unpack(), xs, ws["qkv"].wscale, 1)
-            q, k, v = S.qkv_headnorm_y(y, nw["self_attn.q_norm"], nw["self_attn.k_norm"], self.eps, L, hq, hk, d)
-            o = self._attention(cache[i], q, k, v, L)
+            if cache[i].offset + L > cache[i].k.shape[1]:
+                raise ValueError("KV cache is full")
+            o = self._attend(cache[i], self._qkv(cache[i], L, nw, y=y), L)
             xq, xs = S.act_quant(o, Mp)
             h = S.mm_epi(xq, ws["o"].unpack(), xs, ws["o"].wscale, 2, res=h)
             xq, xs = S.rmsnorm_quant(h, nw["post_attention_layernorm"], self.eps)
@@ -173,9 +176,9 @@ class FusedQwen3:
         xq, xs = S.rmsnorm_quant(h, self.layers[0][0]["input_layernorm"], self.eps, Mp)
         for i, (nw, ws) in enumerate(self.layers):
             acc = S.mm_i8_i32(xq, ws["qkv"].unpack())
-            q, k, v = S.qkv_epilogue_headnorm(acc, xs, ws["qkv"].wscale, nw["self_attn.q_norm"], nw["self_attn.k_norm"],
-                                              self.eps, L, hq, hk, d)
-            o = self._attention(cache[i], q, k, v, L)
+            if cache[i].offset + L > cache[i].k.shape[1]:
+                raise ValueError("KV cache is full")
+            o = self._attend(cache[i], self._qkv(cache[i], L, nw, acc=acc, xs=xs, ws=ws["qkv"].wscale), L)
             xq, xs = S.act_quant(o, Mp)
             acc = S.mm_i8_i32(xq, ws["o"].unpack())
             h, xq, xs = S.res_norm_quant(acc, xs, ws["o"].wscale, h, nw["post_attention_layernorm"], self.eps)
@@ -202,25 +205,38 @@ class DecodeQwen3:
     (e2e/decode.py:29-99).  fuse_prologue="act" (default): RMSNorm + INT8 as separate kernels, the per-token INT8 of
     the o / down inputs inside those GEMVs' prologues; True: every quantization in a GEMV prologue; False: all
     separate.  graphs=True captures the two fixed-shape halves of every layer in HIP graphs on first use;
-    graphs="step" captures the whole step (all layers, attention over the full cache buffer under a position mask,
-    output head) as one graph per cache."""
+    graphs="step" captures the whole step (all layers and the output head) as one graph per cache.  A graph is bound to the cache it was captured with."""
 
     def __init__(self, fused, fuse_prologue="act", graphs=False, head=True):
         assert fused.epilogue == "gemm"
         self.f, self.args, self.fuse, self.head = fused, fused.args, fuse_prologue, head
         self.graphs = {} if graphs else None
         self.whole_step = graphs == "step"
+        self.pos = torch.zeros(1, dtype=torch.int64, device=fused.device)   # position of the token being decoded
+        self.packed_head = None
+        if head == "packed":   # the output projection as SC-MXFP4 too (quantized here, on the device): 4x fewer bytes
+            codes, bc, ws, _ = F.quantize(fused.lm_head, None, with_q=False)
+            self.packed_head = (codes, bc, ws, fused.lm_head.shape[0])
 
-    def _pre(self, h, nw, w):
-        f, a = self.f, self.args
-        hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
+    def _logits(self, h):
+        f = self.f
+        hn = rms_norm(h, f.norm, f.eps)
+        if not self.head:
+            return hn
+        if self.packed_head is None:
+            return f.logits(hn)
+        codes, bc, ws, n = self.packed_head
+        return G.gemv(hn, codes, bc, None, ws, n, 1, pro=1)[None]
+
+    def _pre(self, h, nw, w, c, pos):
+        f = self.f
         if self.fuse is True:
             y = G.gemv(h, w.codes, w.bcodes, None, w.wscale, w.N, 1, pro=2, nw=nw["input_layernorm"], eps=f.eps,
                        fmt=f.fmt)
         else:
             xq, xs = S.rmsnorm_quant(h, nw["input_layernorm"], f.eps, 1)
             y = G.gemv(xq, w.codes, w.bcodes, xs, w.wscale, w.N, 1, fmt=f.fmt)
-        return S.qkv_headnorm_y(y[None], nw["self_attn.q_norm"], nw["self_attn.k_norm"], f.eps, 1, hq, hk, d)
+        return f._qkv(c, 1, nw, y=y[None], pos=pos)
 
     def _post(self, o, h, nw, ws):
         f = self.f
@@ -241,8 +257,8 @@ class DecodeQwen3:
         xq, xs = S.act_quant(act[None], 1)
         return G.gemv(xq, wd.codes, wd.bcodes, xs, wd.wscale, wd.N, 2, res=h, fmt=f.fmt)[None]
 
-    def _graphed(self, key, fn, inputs):
-        """Capture fn(*static inputs) once per key; later calls copy the inputs in and replay."""
+    def _capture(self, key, fn, inputs):
+        """Capture fn(*static copies of inputs) once per key; returns (graph, static inputs, static outputs)."""
         if key not in self.graphs:
             static = [t.clone() for t in inputs]
             s = torch.cuda.Stream()
@@ -254,80 +270,54 @@ class DecodeQwen3:
             with torch.cuda.graph(g):
                 out = fn(*static)
             self.graphs[key] = (g, static, out)
-        g, static, out = self.graphs[key]
+        return self.graphs[key]
+
+    def _replay(self, key, fn, inputs):
+        g, static, out = self._capture(key, fn, inputs)
         for dst, src in zip(static, inputs):
             dst.copy_(src)
         g.replay()
         return out
 
     # ---- the whole step as one HIP graph -----------------------------------------------------------------------
-    # Everything that changes from token to token lives in device memory (token id, position), the KV cache is
-    # written with an index copy at the position and attention runs over the whole cache buffer under a position
-    # mask, so the launch sequence is identical for every token and one graph replay per token replaces
-    # ~25 launches and their host-side preparation per layer.
-    def _step_static(self, tok, pos, cache):
-        f, a = self.f, self.args
-        hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
+    # Everything that changes from token to token lives in device memory (token id, position): the fused
+    # norm + rotary + append kernel and the attention kernel read the position from there, so the launch sequence is
+    # identical for every token and one graph replay per token replaces every launch of the step and its host-side
+    # preparation.
+    def _step_static(self, tok, cache):
+        f = self.f
         h = f.embed.index_select(0, tok)
-        ang = pos.to(torch.float32)[:, None] * f.inv_freq[None]
-        cos, sin = ang.cos()[None], ang.sin()[None]
-
-        def rope(x):
-            x1, x2 = x.float().chunk(2, -1)
-            return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], -1).to(x.dtype)
-        mask = (torch.arange(cache[0].k.shape[1], device=tok.device)[None] <= pos[:, None])[None, None]
         for i, (nw, ws) in enumerate(f.layers):
-            q, k, v = self._pre(h, nw, ws["qkv"])
             c = cache[i]
-            c.k.index_copy_(1, pos, rope(k))
-            c.v.index_copy_(1, pos, v)
-            # the hq / hk query heads that share a KV head take the place of the (length-1) query sequence
-            o = TF.scaled_dot_product_attention(rope(q).view(1, hk, hq // hk, d), c.k[None], c.v[None], attn_mask=mask)
-            h = self._post(o.reshape(1, hq * d), h, nw, ws)
-        hn = rms_norm(h, f.norm, f.eps)
-        return f.logits(hn) if self.head else hn
-
-    def _step_graph(self, tok, cache):
-        key = ("step", id(cache))
-        if key not in self.graphs:
-            st_tok = tok.reshape(-1)[:1].clone()
-            st_pos = torch.zeros(1, dtype=torch.int64, device=tok.device)
-            st_pos.fill_(cache[0].offset)
-            s = torch.cuda.Stream()
-            s.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(s):
-                self._step_static(st_tok, st_pos, cache)      # warm-up outside the capture (writes this token's row)
-            torch.cuda.current_stream().wait_stream(s)
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                out = self._step_static(st_tok, st_pos, cache)
-            self.graphs[key] = (g, st_tok, st_pos, out, cache)
-        g, st_tok, st_pos, out, _ = self.graphs[key]
-        if cache[0].offset >= cache[0].k.shape[1]:
-            raise ValueError("KV cache is full")
-        st_tok.copy_(tok.reshape(-1)[:1])
-        st_pos.fill_(cache[0].offset)
-        g.replay()
-        for c in cache:
-            c.offset += 1
-        return out
+            q = self._pre(h, nw, ws["qkv"], c, self.pos)
+            h = self._post(S.attn_decode(q, c.k, c.v, self.pos), h, nw, ws)
+        return self._logits(h)
 
     def step(self, tok, cache):
         """tok: int64 [1] -> logits [1, V] (or the final hidden row when head is False)."""
         f = self.f
         S.set_format(f.fmt)
+        off = cache[0].offset
+        if off >= cache[0].k.shape[1]:
+            raise ValueError("KV cache is full")
+        tok = tok.reshape(-1)[:1]
+        if self.graphs is not None:
+            self.pos.fill_(off)
         if self.whole_step:
-            return self._step_graph(tok, cache)
-        h = f.embed[tok.reshape(-1)[:1]].contiguous()   # [1, D]
+            out = self._replay(("step", id(cache)), lambda t: self._step_static(t, cache), [tok])
+            for c in cache:
+                c.offset = off + 1
+            return out
+        h = f.embed[tok].contiguous()   # [1, D]
         for i, (nw, ws) in enumerate(f.layers):
+            c = cache[i]
             if self.graphs is None:
-                q, k, v = self._pre(h, nw, ws["qkv"])
+                q = self._pre(h, nw, ws["qkv"], c, off)
             else:
-                q, k, v = self._graphed(("pre", i), lambda x, nw=nw, w=ws["qkv"]: self._pre(x, nw, w), [h])
-            o = f._attention(cache[i], q, k, v, 1)
+                q = self._replay(("pre", i, id(c)), lambda x, nw=nw, w=ws["qkv"], c=c: self._pre(x, nw, w, c, self.pos), [h])
+            o = f._attend(c, q, 1)
             if self.graphs is None:
                 h = self._post(o, h, nw, ws)
             else:
-                h = self._graphed(("post", i), lambda x, r, nw=nw, ws=ws: self._post(x, r, nw, ws), [o, h])
-        hn = rms_norm(h, f.norm, f.eps)
-        return f.logits(hn) if self.head else hn
+                h = self._replay(("post", i), lambda x, r, nw=nw, ws=ws: self._post(x, r, nw, ws), [o, h])
+        return self._logits(h)

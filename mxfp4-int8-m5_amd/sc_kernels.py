@@ -210,6 +210,35 @@ def qkv_headnorm_y(y, qn, kn, eps, L, hq, hk, d, deps=()):
     return _headnorm(None, None, None, y, qn, kn, eps, L, hq, hk, d, y.device)
 
 
+def qkv_headnorm_rope(y, qn, kn, eps, L, hq, hk, d, kcache, vcache, pos, inv_freq, acc=None, xscale=None, wscale=None):
+    """qkv_headnorm_y (or, with acc / xscale / wscale, qkv_epilogue_headnorm) fused with the rotary embedding of q
+    and k and the KV-cache append: returns q [hq, L, d]; k and v go to rows pos..pos+L-1 of kcache / vcache
+    [hk, rows, d].  pos: int, or an int64 device tensor (for graph replay)."""
+    src = y if y is not None else acc
+    q = torch.empty((hq, L, d), dtype=torch.bfloat16, device=src.device)
+    assert kcache.shape == vcache.shape and kcache.shape[0] == hk and kcache.shape[2] == d
+    assert kcache.dtype == torch.bfloat16 and inv_freq.dtype == torch.float32 and inv_freq.numel() == d // 2
+    dev_pos = pos if torch.is_tensor(pos) else None
+    assert dev_pos is None or dev_pos.dtype == torch.int64
+    _lib.call("scmx_qkv_headnorm_rope", _lib.ptr(acc), _lib.ptr(xscale), _lib.ptr(wscale), _lib.ptr(y), _lib.ptr(qn),
+              _lib.ptr(kn), _eps(eps), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache), L, hq, hk, d, _lib.ptr(inv_freq),
+              _lib.ptr(dev_pos), 0 if dev_pos is not None else int(pos), kcache.shape[1], _lib.stream())
+    return q
+
+
+def attn_decode(q, kcache, vcache, n, scale=None):
+    """Single-token attention: q bf16 [hq, 1, d] (or [hq, d]) against caches [hk, rows, d] whose first n rows are valid
+    (n: int, or an int64 device tensor holding the position n - 1, for graph replay) -> bf16 [1, hq * d]."""
+    hq, d = q.shape[0], q.shape[-1]
+    hk, rows, _ = kcache.shape
+    out = torch.empty((1, hq * d), dtype=torch.bfloat16, device=q.device)
+    dev_pos = n if torch.is_tensor(n) else None
+    _lib.call("scmx_attn_decode", _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache), _lib.ptr(dev_pos),
+              0 if dev_pos is not None else int(n), _lib.ptr(out), hq, hk, d, rows,
+              float(scale if scale is not None else d ** -0.5), _lib.stream())
+    return out
+
+
 def qkv_fullnorm_y(y, qn, kn, eps, L, h, d, deps=()):
     """OLMoE: bf16 y [Mp, 3 h d] -> q, k, v [h, L, d] with RMSNorm over the full h*d-wide q and k."""
     q, k, v = (torch.empty((h, L, d), dtype=torch.bfloat16, device=y.device) for _ in range(3))

@@ -160,3 +160,77 @@ def test_whole_step_graph_follows_the_eager_decoder(tiny):
         assert c2[0].offset == j + 1
         assert rel(b, a) < 1e-2, (j, rel(b, a))
     assert rel(c2[1].k[:, :30], c1[1].k[:, :30]) < 1e-2 and float(c2[1].k[:, 30:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("L,pos,from_acc", [(1, 17, False), (70, 0, False), (33, 5, True)])
+def test_fused_headnorm_rope_append_against_separate_ops(L, pos, from_acc):
+    """scmx_qkv_headnorm_rope = qkv_headnorm (pinned bit-exactly elsewhere) + float32 rotary embedding + cache write:
+    q and the written cache rows match the separate ops to bf16 rounding (sin / cos come from different routines);
+    cache rows outside pos..pos+L-1 are untouched; a device-resident position gives the same bits as a host one."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    hq, hk, d, rows = 4, 2, 128, 96
+    g = torch.Generator(device="cuda").manual_seed(L)
+    n = (hq + 2 * hk) * d
+    qn = (1 + 0.1 * torch.randn(d, device="cuda", generator=g)).to(torch.bfloat16)
+    kn = (1 + 0.1 * torch.randn(d, device="cuda", generator=g)).to(torch.bfloat16)
+    inv_freq = 1.0 / (1e4 ** (torch.arange(d // 2, device="cuda", dtype=torch.float32) / (d // 2)))
+    kw = {}
+    if from_acc:
+        acc = torch.randint(-20000, 20000, (L, n), device="cuda", dtype=torch.int32, generator=g)
+        xs, ws = torch.rand(L, device="cuda", generator=g) * 1e-2, torch.rand(n, device="cuda", generator=g) * 1e-2
+        y, kw = None, dict(acc=acc, xscale=xs, wscale=ws)
+        q0, k0, v0 = S.qkv_epilogue_headnorm(acc, xs, ws, qn, kn, 1e-6, L, hq, hk, d)
+    else:
+        y = torch.randn(L, n, device="cuda", generator=g).to(torch.bfloat16)
+        q0, k0, v0 = S.qkv_headnorm_y(y, qn, kn, 1e-6, L, hq, hk, d)
+
+    def rope(x):
+        ang = torch.arange(pos, pos + L, device="cuda", dtype=torch.float32)[:, None] * inv_freq[None]
+        x1, x2 = x.float().chunk(2, -1)
+        return torch.cat([x1 * ang.cos() - x2 * ang.sin(), x2 * ang.cos() + x1 * ang.sin()], -1).to(x.dtype)
+    kc = torch.full((hk, rows, d), 7.0, device="cuda", dtype=torch.bfloat16)
+    vc = torch.full((hk, rows, d), 7.0, device="cuda", dtype=torch.bfloat16)
+    q = S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc, vc, pos, inv_freq, **kw)
+    assert rel(q, rope(q0)) < 4e-3 and rel(kc[:, pos:pos + L], rope(k0)) < 4e-3
+    assert torch.equal(vc[:, pos:pos + L], v0)
+    for c in (kc, vc):
+        assert bool((c[:, :pos] == 7).all()) and bool((c[:, pos + L:] == 7).all())
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2 = S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc2, vc2, torch.tensor([pos], device="cuda"), inv_freq, **kw)
+    assert torch.equal(q2, q) and torch.equal(kc2[:, pos:pos + L], kc[:, pos:pos + L])
+    with pytest.raises(ValueError):
+        S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc, vc, rows - L + 1, inv_freq, **kw)
+
+
+@pytest.mark.parametrize("hq,hk,d,rows,n", [(16, 8, 128, 512, 129), (4, 4, 64, 40, 1), (8, 2, 256, 300, 300),
+                                            (16, 8, 128, 4096, 3000)])
+def test_attn_decode_against_torch(hq, hk, d, rows, n):
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    g = torch.Generator(device="cuda").manual_seed(n)
+    q = torch.randn(hq, 1, d, device="cuda", generator=g).to(torch.bfloat16)
+    kc = torch.randn(hk, rows, d, device="cuda", generator=g).to(torch.bfloat16)
+    vc = torch.randn(hk, rows, d, device="cuda", generator=g).to(torch.bfloat16)
+    rep = hq // hk
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.float()[None], kc[:, :n].float().repeat_interleave(rep, 0)[None], vc[:, :n].float().repeat_interleave(rep, 0)[None])
+    ref = ref[0].transpose(0, 1).reshape(1, hq * d)
+    o = S.attn_decode(q, kc, vc, n)
+    assert o.shape == (1, hq * d) and rel(o, ref) < 6e-3, rel(o, ref)
+    o2 = S.attn_decode(q, kc, vc, torch.tensor([n - 1], device="cuda"))       # position from device memory
+    assert torch.equal(o2, o)
+    with pytest.raises(ValueError):
+        S.attn_decode(q, kc, vc, rows + 1)
+
+
+def test_packed_output_head(tiny):
+    """head="packed": logits through the W4A8 GEMV on the quantized output projection, against the bf16 head."""
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (12,), generator=torch.Generator().manual_seed(7)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    c1, c2 = m.make_cache(32), m.make_cache(32)
+    m.hidden(ids[:11], c1)
+    m.hidden(ids[:11], c2)
+    a = Q.DecodeQwen3(m).step(ids[11:], c1)
+    b = Q.DecodeQwen3(m, head="packed").step(ids[11:], c2)
+    assert b.shape == a.shape and rel(b, a) < 0.15      # 4-bit weights on a 256-wide hidden state
+    assert int(a.argmax()) == int(b.argmax()) or rel(b, a) < 0.1
