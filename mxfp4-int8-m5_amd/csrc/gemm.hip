@@ -28,6 +28,7 @@ struct GemmArgs {
     int bc_row_bytes;
     int epi;
     const int32_t* off;      // grouped: expert segment offsets [E+1]; dense: NULL
+    const uint16_t* silu;    // SwiGLU epilogue: lookup table over bf16 gate values
     const int32_t* tstart;   // grouped: first row tile of each expert [E+1]
     int n_experts;
     DevFormat fmt;
@@ -397,8 +398,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                     y[r] = __fmul_rn(__fmul_rn(float(acc[i][j][4 * g + r]), xs), w4[r]);
                 uint16_t* out = reinterpret_cast<uint16_t*>(a.out);
                 if (epi == SCMX_EPI_SWIGLU) {   // (g, g, u, u) -> two outputs
-                    const uint16_t s0 = swiglu_bf16(round_bf16(y[0]), round_bf16(y[2]));
-                    const uint16_t s1 = swiglu_bf16(round_bf16(y[1]), round_bf16(y[3]));
+                    const uint16_t s0 = swiglu_lut(a.silu, y[0], round_bf16(y[2]));
+                    const uint16_t s1 = swiglu_lut(a.silu, y[1], round_bf16(y[3]));
                     const uint32_t o = uint32_t(s0) | (uint32_t(s1) << 16);
                     if (wide)
                         *reinterpret_cast<uint32_t*>(wtile + row * rsb + col) = o;
@@ -475,7 +476,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
 template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2>
-static void launch_tile(const GemmArgs& a, int bmode, int row_tiles, hipStream_t s) {
+static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStream_t s) {
+    GemmArgs a = a_in;
+    if (a.epi == SCMX_EPI_SWIGLU) a.silu = silu_table_device();
     const int num_n = (a.N + BN - 1) / BN;
     if (a.tstart) row_tiles = (row_tiles + 7) & ~7;   // grouped: whole chunks of 8 row-tile slots (spare slots exit at once)
     const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * 64);
@@ -524,6 +527,10 @@ static int check_gemm_common(const char* who, int M, int N, int K, int epi, bool
     if (epi == SCMX_EPI_SWIGLU && N % 8) {
         set_error("%s: the SwiGLU epilogue needs N %% 8 == 0", who);
         return SCMX_ERR_ARG;
+    }
+    if (epi == SCMX_EPI_SWIGLU && !silu_table_device()) {
+        set_error("%s: the SiLU table of the SwiGLU epilogue could not be located on the device", who);
+        return SCMX_ERR_LAUNCH;
     }
     return SCMX_OK;
 }

@@ -73,6 +73,13 @@ __device__ __forceinline__ uint16_t swiglu_bf16(float g, float u) {
     return f32_to_bf16(__fmul_rn(silu, u));
 }
 
+// Device address (current device) of the 65536-entry table silu[g] = bf16(g * sigmoid(g)) over bf16 gate bit patterns,
+// built at compile time from the same operation sequence as swiglu_bf16; NULL if the symbol cannot be resolved.
+const uint16_t* silu_table_device();
+__device__ __forceinline__ uint16_t swiglu_lut(const uint16_t* __restrict__ table, float g, float u) {
+    return f32_to_bf16(__fmul_rn(bf16_to_f32(table[f32_to_bf16(g)]), u));
+}
+
 // ---- 4-bit code decode -----------------------------------------------------------------------------------------
 // v_perm_b32: byte i of the result is byte sel[i] of the 8-byte value {hi, lo} (selector 0..3 -> lo, 4..7 -> hi).
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {

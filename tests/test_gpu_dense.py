@@ -181,3 +181,33 @@ def test_linear_one_call(S, m, n, k):
     assert np.array_equal(wh[:m * k].view(np.int8).reshape(m, k), xq_ref)
     off = (m * k + 255) & ~255
     assert np.array_equal(wh[off:off + 4 * m].view(np.float32), xs_ref)
+
+
+def test_swiglu_epilogue_every_gate_value(S):
+    """The SwiGLU epilogue looks silu(g) up in a 65536-entry table built at compile time.  Drive every bf16 bit
+    pattern through it as the gate (acc = +-1, xscale = 1, wscale = the value itself) with two different up values
+    and compare with the oracle's operation-by-operation bf16 evaluation: bit-exact for every finite gate, NaN where
+    the oracle gives NaN."""
+    allb = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    gate = bf16.from_bits(allb)                                   # float32 values incl. inf / NaN / denormals
+    n, k = 4 * 32768, 128
+    ws = np.empty(n, F32)
+    ws4 = ws.reshape(-1, 4)
+    ws4[:, 0], ws4[:, 1] = gate[0::2], gate[1::2]
+    ws4[:, 2], ws4[:, 3] = F32(1.0), F32(-0.3984375)              # up values (bf16-representable)
+    code4 = np.zeros((n, k), np.uint8)
+    code4[:, 0] = 1                                               # weight row = (1, 0, 0, ...): acc = xq[:, 0]
+    codes, bc, _ = layout.pack_rows(code4, np.zeros((n, k // 32), np.uint8), ws)
+    xq = np.zeros((2, k), np.int8)
+    xq[0, 0], xq[1, 0] = 1, -1
+    xs = np.ones(2, F32)
+    wq = S.unpack_i8(dev(codes), dev(bc), n, k)
+    got = host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 3))
+    acc = np.stack([np.ones(n, np.int32), -np.ones(n, np.int32)])
+    with np.errstate(all="ignore"):
+        want = linear.epilogue(acc, xs, ws, 3)
+    assert got.shape == want.shape == (2, n // 2)
+    nan = np.isnan(bf16.from_bits(want))
+    assert np.array_equal(np.isnan(bf16.from_bits(got)), nan)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert (~nan).sum() > 2 * 65000
