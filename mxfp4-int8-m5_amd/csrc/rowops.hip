@@ -147,7 +147,8 @@ __global__ __launch_bounds__(NT) void res_norm_quant_kernel(const int32_t* __res
 // ---- swiglu_quant ----------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(NT) void swiglu_quant_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
                                                           const float* __restrict__ wscale, int8_t* __restrict__ xq,
-                                                          float* __restrict__ xs, int F) {
+                                                          float* __restrict__ xs, int F,
+                                                          const uint16_t* __restrict__ silu) {
     extern __shared__ __attribute__((aligned(16))) uint16_t srow[];   // F bf16 + 72 floats
     float* red = reinterpret_cast<float*>(srow + F);
     const int row = blockIdx.x;
@@ -161,9 +162,9 @@ __global__ __launch_bounds__(NT) void swiglu_quant_kernel(const int32_t* __restr
         uint16_t o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float g = round_bf16(__fmul_rn(__fmul_rn(float(g4[i]), xsr), wg[i]));
+            const float g = __fmul_rn(__fmul_rn(float(g4[i]), xsr), wg[i]);
             const float u = round_bf16(__fmul_rn(__fmul_rn(float(u4[i]), xsr), wu[i]));
-            o[i] = swiglu_bf16(g, u);
+            o[i] = swiglu_lut(silu, g, u);   // table over the bf16 value of the gate
         }
         *reinterpret_cast<u32x2*>(srow + 4 * c) =
             u32x2{uint32_t(o[0]) | (uint32_t(o[1]) << 16), uint32_t(o[2]) | (uint32_t(o[3]) << 16)};
@@ -482,7 +483,13 @@ int scmx_swiglu_quant(const int32_t* acc, const float* xscale, const float* wsca
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
-    swiglu_quant_kernel<<<dim3(Mp), dim3(NT), size_t(F) * 2 + 72 * 4, (hipStream_t)stream>>>(acc, xscale, wscale, xq, xs, F);
+    const uint16_t* silu = silu_table_device();
+    if (!silu) {
+        set_error("swiglu_quant: the SiLU table could not be located on the device");
+        return SCMX_ERR_LAUNCH;
+    }
+    swiglu_quant_kernel<<<dim3(Mp), dim3(NT), size_t(F) * 2 + 72 * 4, (hipStream_t)stream>>>(acc, xscale, wscale, xq, xs, F,
+                                                                                            silu);
     return check_launch("swiglu_quant");
 }
 
