@@ -234,3 +234,102 @@ def test_packed_output_head(tiny):
     b = Q.DecodeQwen3(m, head="packed").step(ids[11:], c2)
     assert b.shape == a.shape and rel(b, a) < 0.15      # 4-bit weights on a 256-wide hidden state
     assert int(a.argmax()) == int(b.argmax()) or rel(b, a) < 0.1
+
+
+# ---- OLMoE ---------------------------------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def tiny_moe():
+    from mxfp4_int8_m5_amd import fused_olmoe as O, sc_weights as W
+    args = O.OlmoeArgs(hidden_size=256, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4, num_experts=8,
+                       num_experts_per_tok=2, vocab_size=300)
+    g = torch.Generator().manual_seed(10)
+    rnd = lambda *s, sc=1.0: torch.randn(*s, generator=g) * sc   # noqa: E731
+    D, Fi, E = args.hidden_size, args.intermediate_size, args.num_experts
+    state = {"model.embed_tokens.weight": rnd(args.vocab_size, D), "model.norm.weight": 1 + rnd(D, sc=0.1),
+             "lm_head.weight": rnd(args.vocab_size, D, sc=D ** -0.5)}
+    lin = {}
+    for i in range(2):
+        p = f"model.layers.{i}."
+        for n in ("input_layernorm", "post_attention_layernorm", "self_attn.q_norm", "self_attn.k_norm"):
+            state[p + n + ".weight"] = 1 + rnd(D, sc=0.1)
+        state[p + "mlp.gate.weight"] = rnd(E, D, sc=4 * D ** -0.5)       # a decisive router
+        for n in O.ATTN:
+            lin[f"layers.{i}.{n}"] = rnd(D, D, sc=D ** -0.5)
+        lin[f"layers.{i}.experts.gate_proj"] = rnd(E, Fi, D, sc=D ** -0.5)
+        lin[f"layers.{i}.experts.up_proj"] = rnd(E, Fi, D, sc=D ** -0.5)
+        lin[f"layers.{i}.experts.down_proj"] = rnd(E, D, Fi, sc=Fi ** -0.5)
+    state = {k: v.to(torch.bfloat16).float() for k, v in state.items()}
+    flat = W.pack_weights(lin)
+    packed = {k[:-len(".codes")]: (flat[k], flat[k[:-5] + "bcodes"], flat[k[:-5] + "wscale"]) for k in flat if k.endswith(".codes")}
+    return O, args, state, packed
+
+
+def moe_float_model(args, state, packed, ids, routing):
+    """float32 torch on the CPU with the dequantized weights, no activation quantization, and the routing decisions
+    of the run under test (a near-tie in the router would otherwise send a token to other experts)."""
+    from oracle import layout
+    a = args
+    H, d, eps, E = a.num_attention_heads, a.head_dim, a.rms_norm_eps, a.num_experts
+
+    def weight(key):
+        c, b, s = packed[key]
+        rows = s.shape[0]
+        return torch.from_numpy(layout.decode(c, b, rows, c.size * 8 // rows).astype(np.float32) * s[:, None])
+
+    def norm(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+
+    def rope(x):
+        L, half = x.shape[1], d // 2
+        ang = torch.arange(L, dtype=torch.float32)[:, None] * (1.0 / (a.rope_theta ** (torch.arange(half).float() / half)))[None]
+        x1, x2 = x.chunk(2, -1)
+        return torch.cat([x1 * ang.cos() - x2 * ang.sin(), x2 * ang.cos() + x1 * ang.sin()], -1)
+
+    h = state["model.embed_tokens.weight"][ids]
+    L = h.shape[0]
+    for i in range(a.num_hidden_layers):
+        p, lk = f"model.layers.{i}.", f"layers.{i}."
+        x = norm(h, state[p + "input_layernorm.weight"])
+        q = norm(x @ weight(lk + "self_attn.q_proj").T, state[p + "self_attn.q_norm.weight"]).view(L, H, d).transpose(0, 1)
+        k = norm(x @ weight(lk + "self_attn.k_proj").T, state[p + "self_attn.k_norm.weight"]).view(L, H, d).transpose(0, 1)
+        v = (x @ weight(lk + "self_attn.v_proj").T).view(L, H, d).transpose(0, 1)
+        o = torch.nn.functional.scaled_dot_product_attention(rope(q)[None], rope(k)[None], v[None], is_causal=True)[0]
+        h = h + o.transpose(0, 1).reshape(L, -1) @ weight(lk + "self_attn.o_proj").T
+        x = norm(h, state[p + "post_attention_layernorm.weight"])
+        inds, scores = (t.cpu() for t in routing[i])
+        y = torch.zeros_like(h)
+        for t in range(L):
+            for j in range(inds.shape[1]):
+                e = int(inds[t, j])
+                g = x[t] @ weight(f"{lk}experts.gate_proj.{e}").T
+                u = x[t] @ weight(f"{lk}experts.up_proj.{e}").T
+                y[t] += float(scores[t, j]) * ((torch.nn.functional.silu(g) * u) @ weight(f"{lk}experts.down_proj.{e}").T)
+        h = h + y
+    return norm(h, state["model.norm.weight"])
+
+
+@pytest.mark.parametrize("kw", [dict(tile=64), dict(tile=256, two_pass=True), dict(tile=128, sort="argsort")])
+def test_olmoe_prefill_against_float_model(tiny_moe, kw):
+    O, args, state, packed = tiny_moe
+    ids = torch.randint(0, args.vocab_size, (45,), generator=torch.Generator().manual_seed(11))
+    m = O.FusedOlmoe(args, state, packed, **kw)
+    m.record = []
+    h = m.hidden(ids.cuda())
+    ref = moe_float_model(args, state, packed, ids, m.record)
+    assert rel(h, ref) < 4e-2, rel(h, ref)
+
+
+@pytest.mark.parametrize("fuse", [False, "o", True])
+def test_olmoe_decode_continues_the_prefill(tiny_moe, fuse):
+    O, args, state, packed = tiny_moe
+    ids = torch.randint(0, args.vocab_size, (30,), generator=torch.Generator().manual_seed(12)).cuda()
+    m = O.FusedOlmoe(args, state, packed, tile=64)
+    full = m.hidden(ids)
+    cache = m.make_cache(64)
+    m.hidden(ids[:27], cache)
+    dec = O.DecodeOlmoe(m, fuse_prologue=fuse, head=False)
+    rows = torch.cat([dec.step(ids[27 + j:28 + j], cache) for j in range(3)])
+    assert rel(rows, full[27:]) < 3e-2, rel(rows, full[27:])
+    logits = O.DecodeOlmoe(m).step(ids[:1], m.make_cache(8))
+    assert logits.shape == (1, args.vocab_size)
