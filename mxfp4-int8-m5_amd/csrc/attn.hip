@@ -37,32 +37,39 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
     }
     float m = -3.0e38f, l = 0.0f;
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    // The trip count depends on the group only through "j < n"; every lane of a wave runs the same number of trips
-    // (rows beyond n are skipped by predication), so the cross-lane sums below always see whole groups.
+    // Every lane of the workgroup runs the same number of trips (rows beyond n are skipped by predication), so the
+    // cross-lane sums below always see whole groups.
     const int trips = (n + GROUPS - 1) / GROUPS;
-#pragma unroll 4
-    for (int t = 0; t < trips; ++t) {
-        const int j = t * GROUPS + grp;
-        const bool ok = j < n;
-        const size_t ro = size_t(ok ? j : 0) * D;
-        const u32x4 kw = *reinterpret_cast<const u32x4*>(kbase + ro);
-        const u32x4 vw = *reinterpret_cast<const u32x4*>(vbase + ro);
-        float s = 0.0f;
+    constexpr int UN = 4;   // rows in flight per lane group: the K and V rows of UN steps are requested together
+    for (int t0 = 0; t0 < trips; t0 += UN) {
+        u32x4 kw[UN], vw[UN];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            s += qv[2 * i] * __uint_as_float(kw[i] << 16) + qv[2 * i + 1] * __uint_as_float(kw[i] & 0xFFFF0000u);
+        for (int u = 0; u < UN; ++u) {
+            const int j = (t0 + u) * GROUPS + grp;
+            const size_t ro = size_t(j < n ? j : 0) * D;
+            kw[u] = *reinterpret_cast<const u32x4*>(kbase + ro);
+            vw[u] = *reinterpret_cast<const u32x4*>(vbase + ro);
+        }
 #pragma unroll
-        for (int off = LPR / 2; off >= 1; off >>= 1) s += __shfl_xor(s, off, WAVE);
-        if (ok) {
-            const float mn = fmaxf(m, s);
-            const float alpha = __expf(m - mn), p = __expf(s - mn);
-            l = l * alpha + p;
+        for (int u = 0; u < UN; ++u) {
+            const bool ok = (t0 + u) * GROUPS + grp < n;
+            float s = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[2 * i] = acc[2 * i] * alpha + p * __uint_as_float(vw[i] << 16);
-                acc[2 * i + 1] = acc[2 * i + 1] * alpha + p * __uint_as_float(vw[i] & 0xFFFF0000u);
+            for (int i = 0; i < 4; ++i)
+                s += qv[2 * i] * __uint_as_float(kw[u][i] << 16) + qv[2 * i + 1] * __uint_as_float(kw[u][i] & 0xFFFF0000u);
+#pragma unroll
+            for (int off = LPR / 2; off >= 1; off >>= 1) s += __shfl_xor(s, off, WAVE);
+            if (ok) {
+                const float mn = fmaxf(m, s);
+                const float alpha = __expf(m - mn), p = __expf(s - mn);
+                l = l * alpha + p;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[2 * i] = acc[2 * i] * alpha + p * __uint_as_float(vw[u][i] << 16);
+                    acc[2 * i + 1] = acc[2 * i + 1] * alpha + p * __uint_as_float(vw[u][i] & 0xFFFF0000u);
+                }
+                m = mn;
             }
-            m = mn;
         }
     }
     if (c == 0) {
