@@ -239,3 +239,27 @@ def test_linear_layer_replays_in_a_hip_graph(S):
         want = S.linear_w4a8(xn, dc, db, dw, n)          # eager, own workspace
         torch.cuda.synchronize()
         assert torch.equal(y, want), seed
+
+
+@pytest.mark.parametrize("m,n,k,fmt_i", [(4000, 4096, 256, 0), (4096, 4100, 128, 0), (4096, 4096, 128, 2)])
+def test_widest_tile_configuration(S, m, n, k, fmt_i):
+    """Problems with at least 256 tiles of 256 x 256 run the widest configuration (wave tiles of 128 x 64, K steps of
+    64): ragged last row and column tiles, the published and a generic format, INT32 and all scaling epilogues,
+    bit-exact against the oracle."""
+    fmt = FORMATS[fmt_i]
+    S.set_format(product_format(fmt))
+    rng = np.random.default_rng(m + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k, fmt)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    xs = (rng.random(m) * 0.02).astype(F32)
+    acc = linear.int_gemm(xq, q)
+    wq = S.unpack_i8(dev(codes), dev(bc), n, k)
+    assert np.array_equal(host(S.mm_i8_i32(dev(xq), wq)), acc)
+    assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 1)), linear.epilogue(acc, xs, ws, 1))
+    res = bf16.to_bits(rng.standard_normal((m, n)).astype(F32))
+    assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 2, res=dev(res))),
+                          linear.epilogue(acc, xs, ws, 2, res))
+    if n % 8 == 0:
+        with np.errstate(all="ignore"):
+            assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 3)), linear.epilogue(acc, xs, ws, 3))
+    S.set_format(product_format(layout.DEFAULT))
