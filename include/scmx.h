@@ -180,6 +180,11 @@ int scmx_moe_combine(const uint16_t* y, const int32_t* pos, const uint16_t* scor
                      const uint16_t* res, const uint16_t* w, float eps, uint16_t* h, int8_t* xq, float* xs, int M,
                      int Mp, int K, int topk, void* stream);
 
+/* Randomized Hadamard rotation of every 32-wide block of x T[M, K] (signs f32 [K], +-1; FP32 butterflies, result times
+ * 1/sqrt(32) rounded to T), then per-token INT8 as scmx_act_quant.  K % 32 == 0, K <= 8192.
+ * Replaces rot_quant, e2e/sc_kernels.py:231-275,571-582. */
+int scmx_rot_quant(const uint16_t* x, const float* signs, int8_t* xq, float* xs, int M, int Mp, int K, void* stream);
+
 /* ---- standard MXFP4 interchange --------------------------------------------------------------------------------- */
 
 /* Standard MXFP4 rows (E2M1 nibbles + one E8M0 byte per 32-block, e8m0 [N, K/32]) -> block codes and row scales of

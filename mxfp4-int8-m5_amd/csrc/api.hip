@@ -205,6 +205,67 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(const uint16_t* __r
     if (lane == 0) xs[row] = s;
 }
 
+// ---- rot_quant: randomized Hadamard rotation of every 32-wide block, then per-token INT8 ---------------------------
+// Thread t owns 4 consecutive values; 8 consecutive lanes hold one block.  Butterfly order as in the host
+// formulation: two stages inside the thread, then strides 1, 2, 4 across lanes (lower = lower + upper,
+// upper = lower - upper); the result times 1/sqrt(32) is rounded to bf16 before the row maximum is taken.
+__global__ __launch_bounds__(256) void rot_quant_kernel(const uint16_t* __restrict__ x, const float* __restrict__ signs,
+                                                        int8_t* __restrict__ xq, float* __restrict__ xs, int M, int K) {
+    __shared__ float red[4];
+    constexpr int MAXJ = 8;   // K <= 8192
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int J = K / 1024, rem = K % 1024;   // whole sweeps of 256 threads x 4 values, then a partial one
+    float v[MAXJ + 1][4];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j <= MAXJ; ++j) {
+        const int p = 4 * (j * 256 + tid);
+        const bool in = j < J || (j == J && p < K);
+        if (j > J || (j == J && rem == 0)) break;
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+        if (in && row < M) {
+            const u32x2 w = *reinterpret_cast<const u32x2*>(x + size_t(row) * K + p);
+            const f32x4 sg = *reinterpret_cast<const f32x4*>(signs + p);
+            a0 = __fmul_rn(__uint_as_float(w[0] << 16), sg[0]);
+            a1 = __fmul_rn(__uint_as_float(w[0] & 0xFFFF0000u), sg[1]);
+            a2 = __fmul_rn(__uint_as_float(w[1] << 16), sg[2]);
+            a3 = __fmul_rn(__uint_as_float(w[1] & 0xFFFF0000u), sg[3]);
+        }
+        float b[4] = {__fadd_rn(a0, a1), __fsub_rn(a0, a1), __fadd_rn(a2, a3), __fsub_rn(a2, a3)};
+        float a[4] = {__fadd_rn(b[0], b[2]), __fadd_rn(b[1], b[3]), __fsub_rn(b[0], b[2]), __fsub_rn(b[1], b[3])};
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float c = __shfl_xor(a[i], h, WAVE);
+                a[i] = (tid & h) ? __fsub_rn(c, a[i]) : __fadd_rn(a[i], c);
+            }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[j][i] = round_bf16(__fmul_rn(a[i], 0.17677669529663687f));
+            if (in) amax = fmaxf(amax, fabsf(v[j][i]));
+        }
+    }
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+#pragma unroll
+    for (int j = 0; j <= MAXJ; ++j) {
+        const int p = 4 * (j * 256 + tid);
+        if (j > J || (j == J && rem == 0)) break;
+        if (j < J || p < K) {
+            uint32_t o = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o |= (uint32_t(quant_code(v[j][i], qi)) & 0xFFu) << (8 * i);
+            *reinterpret_cast<uint32_t*>(xq + size_t(row) * K + p) = o;
+        }
+    }
+    if (tid == 0) xs[row] = row < M ? s : 0.0f;
+}
+
 // ---- standard MXFP4 -> block codes + row scale: one wave per row -----------------------------------------------
 __global__ __launch_bounds__(256) void mxfp4_to_sc_kernel(const uint8_t* __restrict__ e8m0,
                                                           uint8_t* __restrict__ bcodes, float* __restrict__ wscale,
@@ -301,6 +362,20 @@ int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int 
         default: act_quant_kernel<<<dim3(Mp), block, 0, st>>>(x, xq, xs, M, K); break;
     }
     return check_launch("act_quant");
+}
+
+int scmx_rot_quant(const uint16_t* x, const float* signs, int8_t* xq, float* xs, int M, int Mp, int K, void* stream) {
+    if (!x || !signs || !xq || !xs || M < 0 || Mp < M || K <= 0 || K % 32 || K > 8192) {
+        set_error("rot_quant: null pointer, Mp < M, or K not a multiple of 32 in 32..8192 (M=%d Mp=%d K=%d)", M, Mp, K);
+        return SCMX_ERR_ARG;
+    }
+    if (uintptr_t(x) % 8 || uintptr_t(signs) % 16 || uintptr_t(xq) % 4) {
+        set_error("rot_quant: x must be 8-byte, signs 16-byte, xq 4-byte aligned");
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    rot_quant_kernel<<<dim3(Mp), dim3(256), 0, (hipStream_t)stream>>>(x, signs, xq, xs, M, K);
+    return check_launch("rot_quant");
 }
 
 int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,

@@ -76,6 +76,24 @@ def act_quant(x, Mp=None, nt=256, deps=()):
     return xq, xs
 
 
+def rot_signs(K):
+    """The sign vector of the block rotation for input width K (one per width, so q/k/v and gate/up share a rotated
+    input); e2e/sc_kernels.py:566-569."""
+    return torch.from_numpy(np.random.default_rng(0).choice([-1.0, 1.0], size=K).astype(np.float32)).cuda()
+
+
+def rot_quant(x, signs, Mp=None, nt=512, deps=()):
+    """x bf16 [M, K] -> (xq int8 [Mp, K], xscale f32 [Mp]): randomized Hadamard rotation of each 32-wide block, then
+    per-token INT8 (e2e/sc_kernels.py:571-582)."""
+    M, K = x.shape
+    Mp = Mp or pad_rows(M)
+    assert x.dtype == torch.bfloat16 and signs.dtype == torch.float32 and signs.numel() == K
+    xq = torch.empty((Mp, K), dtype=torch.int8, device=x.device)
+    xs = torch.empty(Mp, dtype=torch.float32, device=x.device)
+    _lib.call("scmx_rot_quant", _lib.ptr(x), _lib.ptr(signs), _lib.ptr(xq), _lib.ptr(xs), M, Mp, K, _lib.stream())
+    return xq, xs
+
+
 def _gemm(xq, wq, xscale, wscale, epi, res):
     (M, K), N = xq.shape, wq.shape[0]
     assert xq.dtype == torch.int8 and wq.shape[1] == K

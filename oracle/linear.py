@@ -29,6 +29,37 @@ def act_quant(x, mp=None):
     return xq, xs
 
 
+ROT_NORM = F32(0.17677669529663687)   # 1 / sqrt(32), e2e/sc_kernels.py:578
+
+
+def rot_signs(k):
+    """The sign vector of the rotation for input width k (e2e/sc_kernels.py:566-569)."""
+    return np.random.default_rng(0).choice([-1.0, 1.0], size=k).astype(F32)
+
+
+def rot_blocks(x, signs):
+    """Randomized Hadamard rotation of every 32-wide block in FP32 with the butterfly order of the kernel
+    (e2e/sc_kernels.py:231-256): signs, then inside each group of 4 values the stages (x+y, x-y, z+w, z-w) and
+    (x+z, y+w, x-z, y-w), then across the 8 groups of a block the strides 1, 2, 4 with lower = lower + upper and
+    upper = lower - upper; the result times 1/sqrt(32) is rounded to bf16.  x: FP32 [M, K] holding bf16 values."""
+    x = np.asarray(x, F32) * np.asarray(signs, F32)[None, :]
+    m, k = x.shape
+    a = x.reshape(m, k // 32, 8, 4)
+    a = np.stack([a[..., 0] + a[..., 1], a[..., 0] - a[..., 1], a[..., 2] + a[..., 3], a[..., 2] - a[..., 3]], -1)
+    a = np.stack([a[..., 0] + a[..., 2], a[..., 1] + a[..., 3], a[..., 0] - a[..., 2], a[..., 1] - a[..., 3]], -1)
+    t = np.arange(8)
+    for h in (1, 2, 4):
+        c = a[:, :, t ^ h, :]
+        upper = ((t & h) != 0)[None, None, :, None]
+        a = np.where(upper, c - a, a + c).astype(F32)
+    return bf16.rnd((a * ROT_NORM).astype(F32)).reshape(m, k)
+
+
+def rot_quant(x, signs, mp=None):
+    """rot_blocks followed by the per-token INT8 of act_quant (e2e/sc_kernels.py:257-273)."""
+    return act_quant(rot_blocks(x, signs), mp)
+
+
 def act_quant_f64(x):
     """The float64 variant of sim/make_testcase.py:56-58 (xq = clip(rint(x / xscale))); differs from act_quant
     only at rare rounding ties.  Returned for the float reference path."""

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import bf16, layout, linear
-from tests.util import dev, host
+from tests.util import dev, host, llm_acts
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -144,3 +144,17 @@ def test_standard_mxfp4_import(S):
     e8[0, 0] = e8[0].min() + 7
     with pytest.raises(ValueError):
         sc_format.from_mxfp4(dev(nib), dev(e8))
+
+
+@pytest.mark.parametrize("m,mp,k", [(5, 8, 128), (300, 384, 2048), (64, 64, 6144), (17, 17, 1536), (3, 3, 32)])
+def test_rot_quant(m, mp, k):
+    """Block Hadamard rotation + per-token INT8 (e2e/sc_kernels.py:231-275), bit-exact against the oracle's butterfly
+    restatement: codes and scales, zero padding rows."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    rng = np.random.default_rng(m + k)
+    bits, x = llm_acts(rng, m, k)
+    signs = S.rot_signs(k)
+    assert np.array_equal(host(signs), linear.rot_signs(k))
+    xq, xs = S.rot_quant(dev(bits), signs, mp)
+    wq, ws = linear.rot_quant(x, linear.rot_signs(k), mp)
+    assert np.array_equal(host(xq), wq) and np.array_equal(host(xs), ws)

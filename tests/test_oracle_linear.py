@@ -219,3 +219,23 @@ def test_moe_grouped_gemm_matches_per_expert():
     acc = moe.moe_int_gemm(xq, es, wq)
     for i in range(r):
         assert np.array_equal(acc[i], wq[es[i]].astype(np.int64) @ xq[i].astype(np.int64))
+
+
+def test_rot_blocks_is_a_scaled_hadamard_transform():
+    """The butterfly order of rot_blocks (e2e/sc_kernels.py:231-256) is the Sylvester-ordered Walsh-Hadamard transform
+    of each 32-block of x * signs, scaled by 1/sqrt(32): checked against the explicit matrix in float64; an
+    orthonormal transform, so row norms are preserved; a constant block maps onto its first coefficient."""
+    rng = np.random.default_rng(3)
+    x = bf16.rnd(rng.standard_normal((6, 256)).astype(np.float32))
+    signs = linear.rot_signs(256)
+    assert set(np.unique(signs)) == {-1.0, 1.0} and np.array_equal(signs, linear.rot_signs(256))
+    i = np.arange(32)
+    h = (-1.0) ** np.array([[bin(a & b).count("1") for b in i] for a in i])
+    want = ((x * signs).astype(np.float64).reshape(6, 8, 32) @ h.T / np.sqrt(32)).reshape(6, 256)
+    got = linear.rot_blocks(x, signs).astype(np.float64)
+    assert np.abs(got - want).max() <= 2.0 ** -8 * np.abs(want).max()          # one bf16 rounding
+    assert np.allclose(np.linalg.norm(got, axis=1), np.linalg.norm(x, axis=1), rtol=5e-3)
+    ones = linear.rot_blocks(np.ones((1, 32), np.float32), np.ones(32, np.float32))
+    assert ones[0, 0] == bf16.rnd(np.float32(32) * linear.ROT_NORM) and not ones[0, 1:].any()
+    xq, xs = linear.rot_quant(x, signs, 8)
+    assert xq.shape == (8, 256) and not xq[6:].any() and xs[6] == 0 and np.abs(xq[:6]).max() == 127
