@@ -68,6 +68,19 @@ def pack_rows(code4, bcode, wscale, fmt=None):
     return codes, _pack_bcodes(np.asarray(bcode, np.uint8), fmt), np.asarray(wscale, np.float32)
 
 
+def decode_numpy(codes, bcodes, N, K, fmt=None):
+    """Host-side decode of a packed matrix to the INT8 operand q [N, K], for checks and tools (the kernels never
+    call it; the device decode is sc_kernels.unpack_i8).  e2e/sc_format.py:83-90."""
+    fmt = fmt or DEFAULT
+    w = np.asarray(codes, np.uint32).reshape(N, K // 8)
+    c = ((w[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF).reshape(N, K).astype(np.int64)
+    b = np.arange(K // fmt.block)
+    bc = (np.asarray(bcodes, np.uint8)[:, b // fmt.per_byte].astype(np.int64) >> (fmt.bc_bits * (b % fmt.per_byte))) \
+        & ((1 << fmt.bc_bits) - 1)
+    mag = np.asarray(fmt.code_mag, np.int64)[c & 7] * np.repeat(np.asarray(fmt.mult, np.int64)[bc], fmt.block, axis=1)
+    return np.where(c & 8, -mag, mag).astype(np.int8)
+
+
 def from_shift_layout(codes_u32, shifts, wscale, fmt=None):
     """Byte-shift layout (codes, shifts uint8 [N, K/32] in 0..3, wscale) -> packed block codes; no requantization."""
     fmt = fmt or DEFAULT

@@ -103,6 +103,8 @@ def test_host_helpers_match_the_oracle(pkg):
         ws = rng.random(8).astype(np.float32)
         for got, want in zip(F.pack_rows(c4, b, ws, pf), layout.pack_rows(c4, b, ws, ofmt)):
             assert got.dtype == want.dtype and np.array_equal(got, want)
+        assert np.array_equal(F.decode_numpy(*F.pack_rows(c4, b, ws, pf)[:2], 8, 256, pf),
+                              layout.decode(*layout.pack_rows(c4, b, ws, ofmt)[:2], 8, 256, ofmt))
         assert pf.bits_per_weight(4096) == pytest.approx(4 + ofmt.bc_bits / ofmt.block + 32 / 4096)
     with pytest.raises(AssertionError):
         F.Format(block=12)
