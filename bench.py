@@ -323,12 +323,29 @@ def main():
                              "in float64, bit-identical to the host quantizer)", "us": round(us, 1),
                  "gweights_per_s": round(n * k / us / 1e3, 2),
                  "gbps": round(n * k * (2 * 4 + 0.5 + 1.0 / 128) / us / 1e3, 1)}   # the row is read twice
+        from mxfp4_int8_m5_amd import pack_format as PF
+        fam_name = "e2m1/B16/M1..10"
+        PF.pack_matrix(wf[:2048], fam_name)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(5):
+            PF.pack_matrix(wf[:2048], fam_name)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us_f = e0.elapsed_time(e1) / 5 * 1e3
+        quant["family"] = {"workload": f"float32 2048x{k} -> format {fam_name} (8 row bases x 10 block multipliers tried "
+                                       "per block, float32, bit-identical to the host quantizer)", "us": round(us_f, 1),
+                           "gweights_per_s": round(2048 * k / us_f / 1e3, 2)}
         if not a.no_cpu:
             from oracle import layout as olayout
             wh = wf[:256].cpu().numpy().astype(np.float64)
             t0 = time.perf_counter()
             olayout.quantize(wh)
             quant["cpu_oracle_gweights_per_s"] = round(256 * k / (time.perf_counter() - t0) / 1e9, 4)
+            from oracle import family as ofamily
+            t0 = time.perf_counter()
+            ofamily.quantize(wh[:64].astype(np.float32), ofamily.member(fam_name))
+            quant["family"]["cpu_oracle_gweights_per_s"] = round(64 * k / (time.perf_counter() - t0) / 1e9, 5)
         del wf, qc, qb, qw
 
     # ---- whole model: Qwen3-1.7B architecture with random packed weights, prefill and batch-1 decode -----------------

@@ -206,6 +206,15 @@ int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_
 int scmx_quantize_sc(const void* w, int w_is_bf16, int64_t N, int K, int block, uint32_t* codes, uint8_t* bcodes,
                      float* wscale, void* stream);
 
+/* The quantizer of the integer-exact format family w = base[row] * mult[block] * sign * code (float32 decisions): the
+ * largest row base is peak / (max mult * max code); 8 bases per octave below it are tried in descending order, each
+ * with the per-block multiplier of least squared error, and the first strictly best total wins.  fmt gives block (16
+ * or 32), the ascending code magnitudes and multipliers and the block-code width; outputs in fmt's packed layout
+ * with wscale = the row base.  Bit-identical to the host procedure sim/formats.py:64-107 (quantize_mx) followed by
+ * e2e/pack_format.py:44-76 (pack_matrix / pack_parts).  K a multiple of 8 / bc_bits blocks, at most 16384. */
+int scmx_quantize_family(const scmx_format* fmt, const void* w, int w_is_bf16, int64_t N, int K, uint32_t* codes,
+                         uint8_t* bcodes, float* wscale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

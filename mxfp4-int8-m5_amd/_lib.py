@@ -43,6 +43,7 @@ SIGNATURES = {
     "scmx_moe_combine": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_rot_quant": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "scmx_mxfp4_to_sc": (_I, [_P, _P, _P, _P, _L, _L, _P]),
+    "scmx_quantize_family": (_I, [_FMT, _P, _I, _L, _I, _P, _P, _P, _P]),
     "scmx_quantize_sc": (_I, [_P, _I, _L, _I, _I, _P, _P, _P, _P]),
 }
 

@@ -135,3 +135,27 @@ def test_pack_save_load_and_run(SF, tmp_path):
     oq, os_ = linear.act_quant(bf16.from_bits(xb))
     want = linear.epilogue(linear.int_gemm(oq, q), os_, host(pw.wscale), 1)
     assert np.array_equal(y[:m], want)
+
+
+@pytest.mark.parametrize("name", ["e2m1/B16/M1..10", "e2m1/B16/pow2", "e2m1/B32/pow2", "int4/B32/M1..4", "s10/B16/M1..8"])
+def test_family_quantizer_matches_the_oracle(name, golden):
+    """scmx_quantize_family (pack_format.pack_matrix) against the oracle's float32 quantizer of the integer-exact
+    format family + its packer, bit for bit: the golden matrix of the reference's quantizer and LLM-like weights
+    (rows with outlier columns, an all-zero row, a row so small that its bases are denormal)."""
+    from mxfp4_int8_m5_amd import pack_format as P
+    from oracle import family
+    fam = family.member(name)
+    sf = fam.storage()
+    assert product_format(sf) == P.sc_format_of(name)
+    rng = np.random.default_rng(len(name))
+    mats = [golden["fam/w"].astype(F32), llm_weights(rng, 40, 1024).astype(F32)]
+    mats[1][3] = 0
+    mats[1][5] *= F32(1e-36)
+    for w in mats:
+        _, qi, base, scales = family.quantize(w, fam)
+        codes, bc, ws = family.pack_parts(qi, base, scales, sf)
+        dc, db, dw, st = P.pack_matrix(torch.from_numpy(w).cuda(), name)
+        assert st["exact_q"]
+        assert np.array_equal(host(dw), ws)
+        assert np.array_equal(host(db), bc)
+        assert np.array_equal(host(dc).view(np.uint32), codes)
