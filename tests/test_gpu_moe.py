@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import bf16, layout, linear, moe
-from tests.util import FORMATS, dev, host, product_format, random_packed
+from tests.util import FORMATS, dev, host, llm_acts, product_format, random_packed
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -171,3 +171,67 @@ def test_config3_olmoe_shape_property(M):
     pos, tok, es, off, ts, mt = M.route_sort(dev(inds), e, 128)
     acc = host(M.moe_mm(dev(xq), r, dev(codes), dev(bc), dev(ws), off, ts, mt, d, 0, tile=(128, 64, 4)))
     assert np.array_equal(acc, moe.moe_int_gemm(xq, host(es), wq))
+
+
+def test_config4_sparse_moe_full_size(M):
+    """BASELINE config 4 at its real shape: 256 routed experts + one shared expert (index 256), top-8 + shared = 9
+    slots per token, hidden 2048, expert intermediate 512, the 16-element-block power-of-two format; 2048-token
+    prefill through route_sort -> grouped gate|up GEMM (SwiGLU) -> act_quant -> grouped down GEMM, and the batch-1
+    decode as a 9-slot grouped GEMV.  Checks: the sort contract at full size; the grouped outputs of a sample of
+    expert segments (busiest, emptiest non-empty, shared) bit-exact against the oracle; and two size-independent
+    properties over all 18432 rows: the result does not depend on the row tile (64 vs 256), and every row of the
+    grouped GEMM equals the GEMV of that row on its expert."""
+    from mxfp4_int8_m5_amd import sc_decode as G, sc_kernels as S
+    fmt = layout.Format(block=16)
+    pf = product_format(fmt)
+    rng = np.random.default_rng(4)
+    T, E, topk, D, Fi = 2048, 256, 8, 2048, 512
+    E1 = E + 1
+    inds8, _ = skewed_routing(rng, T, E, topk)
+    inds = np.concatenate([inds8, np.full((T, 1), E, np.int32)], 1)            # shared expert appended for every token
+    R = T * (topk + 1)
+    perm = linear.interleave_gate_up(Fi)
+    gu, dn = [], []
+    for _ in range(E1):                                                        # random codes: 257 x (1024x2048 + 2048x512)
+        c4 = rng.integers(0, 16, (2 * Fi, D), dtype=np.uint8)
+        b = rng.integers(0, 4, (2 * Fi, D // 16), dtype=np.uint8)
+        gu.append(layout.pack_rows(c4[perm], b[perm], np.exp2(rng.integers(-12, -6, 2 * Fi)).astype(F32), fmt))
+        c4 = rng.integers(0, 16, (D, Fi), dtype=np.uint8)
+        b = rng.integers(0, 4, (D, Fi // 16), dtype=np.uint8)
+        dn.append(layout.pack_rows(c4, b, np.exp2(rng.integers(-12, -6, D)).astype(F32), fmt))
+    gc, gb, gw = (dev(np.stack([p[i] for p in gu])) for i in range(3))
+    dc, db, dw = (dev(np.stack([p[i] for p in dn])) for i in range(3))
+    xb, x = llm_acts(rng, T, D)
+    xq, xs = S.act_quant(dev(xb), Mp=T)
+    outs = {}
+    for tm in (64, 256):
+        pos, tok, es, off, ts, mt = M.route_sort(dev(inds), E1, tm)
+        moe.check_route_sort(inds, E1, tm, host(pos), host(tok), host(es), host(off), host(ts))
+        act = M.moe_mm(xq, R, gc, gb, gw, off, ts, mt, 2 * Fi, 3, xs, tile=(tm, 64, 4), gather=tok, fmt=pf)
+        aq, as_ = S.act_quant(act, Mp=R)
+        yd = M.moe_mm(aq, R, dc, db, dw, off, ts, mt, D, 1, as_, tile=(tm, 64, 4), fmt=pf)
+        # rows back in assignment order, so that the comparison does not depend on the order inside the segments
+        outs[tm] = (host(act)[host(pos)], host(yd)[host(pos)])
+    assert np.array_equal(outs[64][0], outs[256][0]) and np.array_equal(outs[64][1], outs[256][1])
+    # oracle on a sample of experts
+    pos_h, off_h, tok_h = host(pos), host(off), host(tok)[:R]
+    counts = np.diff(off_h)
+    assert counts[E] == T and counts.sum() == R
+    rq, rs = linear.act_quant(x)
+    act_h, yd_h, aq_h, as_h = host(act), host(yd), host(aq), host(as_)
+    for e in (int(np.argmax(counts[:E])), int(np.argmin(np.where(counts > 0, counts, R))), E):
+        rows = slice(off_h[e], off_h[e + 1])
+        t = tok_h[rows]
+        q_gu = layout.decode(gu[e][0], gu[e][1], 2 * Fi, D, fmt)
+        a_ref = linear.epilogue(linear.int_gemm(rq[t], q_gu), rs[t], gu[e][2], 3)
+        assert np.array_equal(act_h[rows], a_ref)
+        q2, s2 = linear.act_quant(bf16.from_bits(a_ref))
+        assert np.array_equal(aq_h[rows], q2) and np.array_equal(as_h[rows], s2)
+        q_dn = layout.decode(dn[e][0], dn[e][1], D, Fi, fmt)
+        assert np.array_equal(yd_h[rows], linear.epilogue(linear.int_gemm(q2, q_dn), s2, dn[e][2], 1))
+    # batch-1 decode of token 0: 8 routed slots + the shared expert, one launch per projection
+    eidx = dev(inds8[0].astype(np.int32))
+    a1 = G.gemv(xq[:1], gc, gb, xs[:1], gw, 2 * Fi, 3, eidx=eidx, xstride=0, shared=E, fmt=pf)          # [9, 512]
+    y1 = G.gemv(a1, dc, db, None, dw, D, 1, eidx=eidx, xstride=1, pro=1, shared=E, fmt=pf)              # [9, 2048]
+    mine = pos_h[:topk + 1]                                                    # sorted rows of token 0's assignments
+    assert np.array_equal(host(a1), act_h[mine]) and np.array_equal(host(y1), yd_h[mine])
