@@ -263,3 +263,19 @@ def test_widest_tile_configuration(S, m, n, k, fmt_i):
         with np.errstate(all="ignore"):
             assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 3)), linear.epilogue(acc, xs, ws, 3))
     S.set_format(product_format(layout.DEFAULT))
+
+
+@pytest.mark.parametrize("name,n,k", [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)])
+def test_config1_m8192_and_m512_equal_row_blocks_of_m2048(S, name, n, k):
+    """BASELINE config 1's other token counts.  A row of the output depends on its own activation row only, so the
+    M = 8192 launch (widest tiles) and the M = 512 launches (narrow tiles) must reproduce, bit for bit, the rows that
+    M = 2048 launches (checked against the oracle above) give for the same activations."""
+    rng = np.random.default_rng(n + k)
+    codes, bc, ws, _ = random_packed(rng, n, k)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    x = torch.randn((8192, k), device="cuda", generator=torch.Generator(device="cuda").manual_seed(n)).to(torch.bfloat16)
+    big = S.linear_w4a8(x, dc, db, dw, n)
+    for r0 in range(0, 8192, 2048):
+        assert torch.equal(big[r0:r0 + 2048], S.linear_w4a8(x[r0:r0 + 2048].contiguous(), dc, db, dw, n)), (name, r0)
+    for r0 in (0, 3584):
+        assert torch.equal(big[r0:r0 + 512], S.linear_w4a8(x[r0:r0 + 512].contiguous(), dc, db, dw, n)), (name, r0)
