@@ -499,7 +499,11 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
 static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     const long cus = 256;
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-    if (tiles(256, 256) >= cus) return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
+    // the widest tile only where its tiles fill whole rounds of the 256 CUs (a last round that is mostly empty costs
+    // more than the narrower tile's extra LDS traffic: 384 tiles would take 2 rounds of double-size work)
+    const long t256 = tiles(256, 256);
+    if (t256 >= cus && t256 * 100 >= ((t256 + cus - 1) / cus) * cus * 88)
+        return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
     if (tiles(256, 128) >= cus) return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
     if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
     if (tiles(256, 64) >= cus) return launch_tile<256, 64, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
