@@ -193,6 +193,12 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
     const int heads = hq + 2 * hk, ntot = heads * d, per = d / 64;
     const int64_t pos = rope.inv_freq ? (rope.pos_dev ? rope.pos_dev[0] : rope.pos0) + row : row;
     const int kv_rows = rope.inv_freq ? rope.kv_rows : L;
+    // the d / 2 rotation angles of this row are the same for every head: one sine / cosine each per workgroup
+    __shared__ float s_sin[256], s_cos[256];
+    if (rope.inv_freq) {
+        for (int i = threadIdx.x; i < d / 2; i += NT) sincosf(float(pos) * rope.inv_freq[i], &s_sin[i], &s_cos[i]);
+        __syncthreads();
+    }
     // blockIdx.y strides over groups of NT / 64 heads (one per wave): a single row still fills many CUs
     for (int g = blockIdx.y * (NT / 64) + wave; g < heads; g += gridDim.y * (NT / 64)) {
         float yv[8];   // per <= 8 (d <= 512)
@@ -220,8 +226,7 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
                     // element e = per*lane + i pairs with e +- d/2, held by lane +- 32 at the same i
                     const float other = __shfl_xor(nv, 32, WAVE);
                     const int e = per * lane + i;
-                    float sn, cs;
-                    sincosf(float(pos) * rope.inv_freq[e % (d / 2)], &sn, &cs);
+                    const float sn = s_sin[e % (d / 2)], cs = s_cos[e % (d / 2)];
                     nv = lane < 32 ? __fsub_rn(__fmul_rn(nv, cs), __fmul_rn(other, sn))
                                    : __fadd_rn(__fmul_rn(nv, cs), __fmul_rn(other, sn));
                 }

@@ -85,6 +85,7 @@ class FusedQwen3:
             ws = {g: PackedWeight([packed[f"layers.{i}.{path}"] for path in paths], resident, perm.get(g), self.fmt,
                                   device) for g, paths in GROUPS.items()}
             self.layers.append((norms, ws))
+        self.sdpa_gqa = True    # let the attention op share KV heads between query heads instead of copying them
         half = args.head_dim // 2
         self.inv_freq = 1.0 / (args.rope_theta ** (torch.arange(half, device=device, dtype=torch.float32) / half))
 
@@ -122,14 +123,15 @@ class FusedQwen3:
         hq, hk = q.shape[0], k.shape[0]
         if L == 1:
             return S.attn_decode(q, c.k, c.v, off + 1)
-        if hq != hk:
+        gqa = {"enable_gqa": True} if hq != hk and self.sdpa_gqa else {}
+        if hq != hk and not self.sdpa_gqa:
             k, v = k.repeat_interleave(hq // hk, 0), v.repeat_interleave(hq // hk, 0)
         if off == 0:
-            o = TF.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)
+            o = TF.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True, **gqa)
         else:
             pos = torch.arange(off, off + L, device=q.device)[:, None]
             mask = torch.arange(off + L, device=q.device)[None] <= pos
-            o = TF.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask)
+            o = TF.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask, **gqa)
         return o[0].transpose(0, 1).reshape(L, -1).contiguous()
 
     def _embed(self, ids):
