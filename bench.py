@@ -192,6 +192,29 @@ def main():
                 "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their average launch "
                         "durations, activations pre-quantized", "per_shape": per_shape}
 
+    # ---- the ROCm library's INT8 GEMM on the same shapes: what tuned vendor code reaches here with resident INT8 ----
+    # weights, INT32 output, no unpack and no epilogue (a reference point for the fraction of peak, not a baseline)
+    library = {}
+    if not a.no_sweep:
+        try:
+            for name, n, k in LAYERS:
+                xa = torch.randint(-127, 128, (M_TOKENS, k), dtype=torch.int8, device=dev)
+                wb = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev).t()
+                for _ in range(3):
+                    torch._int_mm(xa, wb)
+                torch.cuda.synchronize()
+                e0.record(stream)
+                for _ in range(20):
+                    torch._int_mm(xa, wb)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / 20
+                library[name] = {"us": round(ms * 1e3, 2), "tops": round(2.0 * M_TOKENS * n * k / ms / 1e9, 1)}
+                del xa, wb
+            library["what"] = "torch._int_mm at M = %d: INT8 x INT8 -> INT32, weights already INT8, no epilogue" % M_TOKENS
+        except Exception as exc:   # the comparison is optional: a build of torch without this op must not stop the bench
+            library = {"error": str(exc)[:200]}
+
     # ---- prefill sweep over M (config 1's other token counts): GEMM kernel alone, per shape ---------------------------
     sweep = {}
     if not a.no_sweep:
@@ -420,6 +443,7 @@ def main():
         "pct_int8_peak": round(tops / PEAK_INT8_TOPS * 100, 2),
         "roofline": roofline,
         "prefill_sweep": sweep,
+        "library_int8_gemm": library,
         "moe": moe,
         "decode": decode,
         "quantize": quant,
