@@ -131,6 +131,15 @@ int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float*
 int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, const int64_t* pos_dev, int n,
                      uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, void* stream);
 
+/* scmx_qkv_headnorm_rope at L = 1 and scmx_attn_decode in one launch: y bf16 [(hq + 2 hk) * d] is the token's q|k|v
+ * row from the qkv projection; per-head RMSNorm of q and k, rotary embedding at position p (*pos_dev, or pos0 when
+ * pos_dev is NULL), append of k and v to row p of the caches, attention over rows 0..p.  Same bits as the two calls.
+ * One launch less per block of the batch-1 decode step (e2e/decode.py:51-82; the array ops it stands for are
+ * e2e/fused_qwen3.py:216-222). */
+int scmx_attn_decode_qkv(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, const float* inv_freq,
+                         const int64_t* pos_dev, int64_t pos0, uint16_t* kcache, uint16_t* vcache, uint16_t* out,
+                         int hq, int hk, int d, int cache_rows, float scale, void* stream);
+
 /* OLMoE q/k/v split with RMSNorm over the full h*d width.  Replaces qkv_fullnorm_y, e2e/sc_kernels.py:390-423,
  * 629-637. */
 int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q,

@@ -12,23 +12,72 @@ namespace scmx {
 
 constexpr int ANT = 256;
 
-template <int D>
-__global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
-                                                         const uint16_t* __restrict__ vc,
+// What the fused variant needs besides the attention operands: the token's q|k|v row as the qkv projection wrote it,
+// the per-head norm weights and the rotary frequencies.
+struct QkvArgs {
+    const uint16_t* y;        // bf16 [(hq + 2 hk) * d]: q heads, k heads, v heads
+    const uint16_t* qn;       // bf16 [d]
+    const uint16_t* kn;       // bf16 [d]
+    const float* inv_freq;    // [d / 2]
+    float eps;
+};
+
+// FUSED: the workgroup first normalises and rotates its own q head and its KV head's new k (as the row kernel
+// qkv_headnorm_kernel does, same arithmetic), keeps them and the new v in LDS, and attends over the cache rows below
+// the position plus that new row; the first query head of every KV group appends the new k and v to the cache.  No
+// workgroup reads what another writes in the same launch.
+template <int D, bool FUSED>
+__global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __restrict__ q, uint16_t* __restrict__ kc,
+                                                         uint16_t* __restrict__ vc,
                                                          const int64_t* __restrict__ pos_dev, int n0,
-                                                         uint16_t* __restrict__ out, int hq, int hk, int rows, float scale) {
+                                                         uint16_t* __restrict__ out, int hq, int hk, int rows, float scale,
+                                                         const QkvArgs x) {
     constexpr int LPR = D / 8;              // lanes per cache row
     constexpr int GROUPS = ANT / LPR;       // lane groups per workgroup, each walking its own rows
     __shared__ float s_m[GROUPS], s_l[GROUPS], s_acc[GROUPS][D];
+    __shared__ float s_sin[FUSED ? D / 2 : 1], s_cos[FUSED ? D / 2 : 1];
+    __shared__ __attribute__((aligned(16))) uint16_t s_new[FUSED ? 3 : 1][D];   // this token's q, k, v (bf16)
     const int n = min(rows, pos_dev ? int(pos_dev[0]) + 1 : n0);
     const int head = blockIdx.x, kvh = head / (hq / hk);
     const int tid = threadIdx.x, grp = tid / LPR, c = tid % LPR;
     const uint16_t* kbase = kc + size_t(kvh) * rows * D + 8 * c;
     const uint16_t* vbase = vc + size_t(kvh) * rows * D + 8 * c;
 
+    if (FUSED) {
+        constexpr int PER = D / 64;
+        const int lane = tid & 63, wave = tid >> 6;
+        const int newrow = n - 1;   // the position of the token being decoded
+        for (int i = tid; i < D / 2; i += ANT) sincosf(float(int64_t(newrow)) * x.inv_freq[i], &s_sin[i], &s_cos[i]);
+        __syncthreads();
+        if (wave < 3) {   // wave 0: q head, wave 1: k head, wave 2: v head
+            const int g = wave == 0 ? head : (wave == 1 ? hq + kvh : hq + hk + kvh);
+            float yv[PER];
+            float ss = 0.0f;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                yv[i] = bf16_to_f32(x.y[size_t(g) * D + PER * lane + i]);
+                ss = __fadd_rn(ss, __fmul_rn(yv[i], yv[i]));
+            }
+            const bool append = wave > 0 && head % (hq / hk) == 0;
+            uint16_t* dst = (wave == 1 ? kc : vc) + (size_t(kvh) * rows + newrow) * D + PER * lane;
+            auto emit = [&](int i, uint16_t b) {
+                s_new[wave][PER * lane + i] = b;
+                if (append) dst[i] = b;
+            };
+            if (wave < 2) {
+                head_norm_rope(yv, ss, PER, lane, D, wave == 0 ? x.qn : x.kn, x.eps, s_sin, s_cos, emit);
+            } else {
+#pragma unroll
+                for (int i = 0; i < PER; ++i) emit(i, f32_to_bf16(yv[i]));
+            }
+        }
+        __syncthreads();
+    }
+
     float qv[8];
     {
-        const u32x4 w = *reinterpret_cast<const u32x4*>(q + size_t(head) * D + 8 * c);
+        const u32x4 w = FUSED ? *reinterpret_cast<const u32x4*>(&s_new[0][8 * c])
+                              : *reinterpret_cast<const u32x4*>(q + size_t(head) * D + 8 * c);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             qv[2 * i] = __uint_as_float(w[i] << 16) * scale;
@@ -46,9 +95,14 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int j = (t0 + u) * GROUPS + grp;
-            const size_t ro = size_t(j < n ? j : 0) * D;
-            kw[u] = *reinterpret_cast<const u32x4*>(kbase + ro);
-            vw[u] = *reinterpret_cast<const u32x4*>(vbase + ro);
+            if (FUSED && j == n - 1) {   // the new row comes from LDS, not from the cache being appended to
+                kw[u] = *reinterpret_cast<const u32x4*>(&s_new[1][8 * c]);
+                vw[u] = *reinterpret_cast<const u32x4*>(&s_new[2][8 * c]);
+            } else {
+                const size_t ro = size_t(j < n ? j : 0) * D;
+                kw[u] = *reinterpret_cast<const u32x4*>(kbase + ro);
+                vw[u] = *reinterpret_cast<const u32x4*>(vbase + ro);
+            }
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
@@ -95,31 +149,68 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
     }
 }
 
+template <bool FUSED>
+static void launch_attn(int d, hipStream_t st, const uint16_t* q, uint16_t* kc, uint16_t* vc, const int64_t* pos_dev, int n,
+                        uint16_t* out, int hq, int hk, int rows, float scale, const QkvArgs& x) {
+    const dim3 grid(hq), wg(ANT);
+    if (d == 64)
+        attn_decode_kernel<64, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x);
+    else if (d == 128)
+        attn_decode_kernel<128, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x);
+    else
+        attn_decode_kernel<256, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x);
+}
+
 }  // namespace scmx
 
 using namespace scmx;
 
-extern "C" int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, const int64_t* pos_dev,
-                                int n, uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, void* stream) {
-    if (!q || !kcache || !vcache || !out || hq < 1 || hk < 1 || hq % hk || cache_rows < 1) {
-        set_error("attn_decode: null pointer or bad head counts (hq=%d hk=%d)", hq, hk);
+static int check_attn(const char* who, int hq, int hk, int d, int cache_rows) {
+    if (hq < 1 || hk < 1 || hq % hk || cache_rows < 1) {
+        set_error("%s: bad head counts or cache size (hq=%d hk=%d rows=%d)", who, hq, hk, cache_rows);
         return SCMX_ERR_ARG;
     }
     if (d != 64 && d != 128 && d != 256) {
-        set_error("attn_decode: head dim must be 64, 128 or 256 (d=%d)", d);
+        set_error("%s: head dim must be 64, 128 or 256 (d=%d)", who, d);
         return SCMX_ERR_ARG;
     }
+    return SCMX_OK;
+}
+
+extern "C" int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, const int64_t* pos_dev,
+                                int n, uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, void* stream) {
+    if (!q || !kcache || !vcache || !out) {
+        set_error("attn_decode: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (int rc = check_attn("attn_decode", hq, hk, d, cache_rows)) return rc;
     if (!pos_dev && (n < 1 || n > cache_rows)) {
         set_error("attn_decode: %d valid rows outside 1..%d", n, cache_rows);
         return SCMX_ERR_ARG;
     }
-    hipStream_t st = (hipStream_t)stream;
-    const dim3 grid(hq), wg(ANT);
-    if (d == 64)
-        attn_decode_kernel<64><<<grid, wg, 0, st>>>(q, kcache, vcache, pos_dev, n, out, hq, hk, cache_rows, scale);
-    else if (d == 128)
-        attn_decode_kernel<128><<<grid, wg, 0, st>>>(q, kcache, vcache, pos_dev, n, out, hq, hk, cache_rows, scale);
-    else
-        attn_decode_kernel<256><<<grid, wg, 0, st>>>(q, kcache, vcache, pos_dev, n, out, hq, hk, cache_rows, scale);
+    launch_attn<false>(d, (hipStream_t)stream, q, const_cast<uint16_t*>(kcache), const_cast<uint16_t*>(vcache), pos_dev, n,
+                       out, hq, hk, cache_rows, scale, QkvArgs{});
     return check_launch("attn_decode");
+}
+
+extern "C" int scmx_attn_decode_qkv(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps,
+                                    const float* inv_freq, const int64_t* pos_dev, int64_t pos0, uint16_t* kcache,
+                                    uint16_t* vcache, uint16_t* out, int hq, int hk, int d, int cache_rows, float scale,
+                                    void* stream) {
+    if (!y || !qn || !kn || !inv_freq || !kcache || !vcache || !out) {
+        set_error("attn_decode_qkv: null pointer argument");
+        return SCMX_ERR_ARG;
+    }
+    if (int rc = check_attn("attn_decode_qkv", hq, hk, d, cache_rows)) return rc;
+    if (uintptr_t(kcache) % 16 || uintptr_t(vcache) % 16) {
+        set_error("attn_decode_qkv: caches must be 16-byte aligned");
+        return SCMX_ERR_ARG;
+    }
+    if (!pos_dev && (pos0 < 0 || pos0 >= cache_rows)) {
+        set_error("attn_decode_qkv: position %lld outside a cache of %d rows", (long long)pos0, cache_rows);
+        return SCMX_ERR_ARG;
+    }
+    launch_attn<true>(d, (hipStream_t)stream, nullptr, kcache, vcache, pos_dev, int(pos0) + 1, out, hq, hk, cache_rows, scale,
+                      QkvArgs{y, qn, kn, inv_freq, eps});
+    return check_launch("attn_decode_qkv");
 }

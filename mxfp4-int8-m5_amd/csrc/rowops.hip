@@ -217,21 +217,8 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
         uint16_t* o = g < hq ? out + (size_t(hh) * L + row) * d + per * lane
                              : out + (size_t(hh) * kv_rows + size_t(pos)) * d + per * lane;
         if (g < hq + hk) {
-            ss = wave_sum(ss);
-            const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
-            const uint16_t* w = g < hq ? qn : kn;
-            for (int i = 0; i < per; ++i) {
-                float nv = round_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
-                if (rope.inv_freq) {
-                    // element e = per*lane + i pairs with e +- d/2, held by lane +- 32 at the same i
-                    const float other = __shfl_xor(nv, 32, WAVE);
-                    const int e = per * lane + i;
-                    const float sn = s_sin[e % (d / 2)], cs = s_cos[e % (d / 2)];
-                    nv = lane < 32 ? __fsub_rn(__fmul_rn(nv, cs), __fmul_rn(other, sn))
-                                   : __fadd_rn(__fmul_rn(nv, cs), __fmul_rn(other, sn));
-                }
-                o[i] = f32_to_bf16(nv);
-            }
+            head_norm_rope(yv, ss, per, lane, d, g < hq ? qn : kn, eps, rope.inv_freq ? s_sin : nullptr, s_cos,
+                           [&](int i, uint16_t b) { o[i] = b; });
         } else {
             for (int i = 0; i < per; ++i) o[i] = f32_to_bf16(yv[i]);
         }

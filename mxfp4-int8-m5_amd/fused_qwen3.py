@@ -207,11 +207,14 @@ class DecodeQwen3:
     (e2e/decode.py:29-99).  fuse_prologue="act" (default): RMSNorm + INT8 as separate kernels, the per-token INT8 of
     the o / down inputs inside those GEMVs' prologues; True: every quantization in a GEMV prologue; False: all
     separate.  graphs=True captures the two fixed-shape halves of every layer in HIP graphs on first use;
-    graphs="step" captures the whole step (all layers and the output head) as one graph per cache.  A graph is bound to the cache it was captured with."""
+    graphs="step" captures the whole step (all layers and the output head) as one graph per cache.  A graph is bound
+    to the cache it was captured with.  fuse_attn=True (default): q/k norm, rotary embedding, cache append and the
+    attention in one kernel; False: two kernels (same bits)."""
 
-    def __init__(self, fused, fuse_prologue="act", graphs=False, head=True):
+    def __init__(self, fused, fuse_prologue="act", graphs=False, head=True, fuse_attn=True):
         assert fused.epilogue == "gemm"
         self.f, self.args, self.fuse, self.head = fused, fused.args, fuse_prologue, head
+        self.fuse_attn = fuse_attn
         self.graphs = {} if graphs else None
         self.whole_step = graphs == "step"
         self.pos = torch.zeros(1, dtype=torch.int64, device=fused.device)   # position of the token being decoded
@@ -238,7 +241,18 @@ class DecodeQwen3:
         else:
             xq, xs = S.rmsnorm_quant(h, nw["input_layernorm"], f.eps, 1)
             y = G.gemv(xq, w.codes, w.bcodes, xs, w.wscale, w.N, 1, fmt=f.fmt)
+        if self.fuse_attn:   # the attention output, not q: the token's k and v are in the cache afterwards
+            a = self.args
+            return S.attn_decode_qkv(y, nw["self_attn.q_norm"], nw["self_attn.k_norm"], f.eps, a.num_attention_heads,
+                                     a.num_key_value_heads, a.head_dim, c.k, c.v, pos, f.inv_freq)
         return f._qkv(c, 1, nw, y=y[None], pos=pos)
+
+    def _attn(self, c, q):
+        """The attention output of the token whose q (or, fused, whose finished attention) _pre returned."""
+        if not self.fuse_attn:
+            return self.f._attend(c, q, 1)
+        c.offset += 1
+        return q
 
     def _post(self, o, h, nw, ws):
         f = self.f
@@ -292,7 +306,7 @@ class DecodeQwen3:
         for i, (nw, ws) in enumerate(f.layers):
             c = cache[i]
             q = self._pre(h, nw, ws["qkv"], c, self.pos)
-            h = self._post(S.attn_decode(q, c.k, c.v, self.pos), h, nw, ws)
+            h = self._post(q if self.fuse_attn else S.attn_decode(q, c.k, c.v, self.pos), h, nw, ws)
         return self._logits(h)
 
     def step(self, tok, cache):
@@ -317,7 +331,7 @@ class DecodeQwen3:
                 q = self._pre(h, nw, ws["qkv"], c, off)
             else:
                 q = self._replay(("pre", i, id(c)), lambda x, nw=nw, w=ws["qkv"], c=c: self._pre(x, nw, w, c, self.pos), [h])
-            o = f._attend(c, q, 1)
+            o = self._attn(c, q)
             if self.graphs is None:
                 h = self._post(o, h, nw, ws)
             else:

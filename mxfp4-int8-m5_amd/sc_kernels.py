@@ -257,6 +257,22 @@ def attn_decode(q, kcache, vcache, n, scale=None):
     return out
 
 
+def attn_decode_qkv(y, qn, kn, eps, hq, hk, d, kcache, vcache, pos, inv_freq, scale=None):
+    """qkv_headnorm_rope at L = 1 followed by attn_decode, in one launch and with the same bits: y bf16
+    [1, (hq + 2 hk) d] -> bf16 [1, hq * d]; the token's k and v land in row pos of the caches.  pos: int, or an int64
+    device tensor (for graph replay)."""
+    assert kcache.shape == vcache.shape and kcache.shape[0] == hk and kcache.shape[2] == d
+    assert y.dtype == torch.bfloat16 and y.numel() == (hq + 2 * hk) * d and kcache.dtype == torch.bfloat16
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == d // 2
+    out = torch.empty((1, hq * d), dtype=torch.bfloat16, device=y.device)
+    dev_pos = pos if torch.is_tensor(pos) else None
+    assert dev_pos is None or dev_pos.dtype == torch.int64
+    _lib.call("scmx_attn_decode_qkv", _lib.ptr(y), _lib.ptr(qn), _lib.ptr(kn), _eps(eps), _lib.ptr(inv_freq),
+              _lib.ptr(dev_pos), 0 if dev_pos is not None else int(pos), _lib.ptr(kcache), _lib.ptr(vcache), _lib.ptr(out),
+              hq, hk, d, kcache.shape[1], float(scale if scale is not None else d ** -0.5), _lib.stream())
+    return out
+
+
 def qkv_fullnorm_y(y, qn, kn, eps, L, h, d, deps=()):
     """OLMoE: bf16 y [Mp, 3 h d] -> q, k, v [h, L, d] with RMSNorm over the full h*d-wide q and k."""
     q, k, v = (torch.empty((h, L, d), dtype=torch.bfloat16, device=y.device) for _ in range(3))

@@ -222,6 +222,51 @@ def test_attn_decode_against_torch(hq, hk, d, rows, n):
         S.attn_decode(q, kc, vc, rows + 1)
 
 
+@pytest.mark.parametrize("hq,hk,d,rows,pos", [(16, 8, 128, 512, 128), (4, 4, 64, 40, 0), (8, 2, 256, 300, 299),
+                                               (32, 8, 128, 2048, 1500), (6, 3, 128, 64, 31)])
+def test_attn_decode_qkv_equals_the_two_kernels(hq, hk, d, rows, pos):
+    """Norm + rotary + append + attention in one launch: the attention output and the appended cache rows carry the
+    same bits as qkv_headnorm_rope followed by attn_decode, with the position as an argument and from device memory;
+    no other cache row is touched."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    g = torch.Generator(device="cuda").manual_seed(pos + d)
+    y = (torch.randn(1, (hq + 2 * hk) * d, device="cuda", generator=g) * 2).to(torch.bfloat16)
+    qn = (1 + 0.1 * torch.randn(d, device="cuda", generator=g)).to(torch.bfloat16)
+    kn = (1 + 0.1 * torch.randn(d, device="cuda", generator=g)).to(torch.bfloat16)
+    inv_freq = (1e6 ** (-torch.arange(0, d, 2, dtype=torch.float32) / d)).cuda()
+    kc = torch.randn(hk, rows, d, device="cuda", generator=g).to(torch.bfloat16)
+    vc = torch.randn(hk, rows, d, device="cuda", generator=g).to(torch.bfloat16)
+    k1, v1, k2, v2, k3, v3 = kc.clone(), vc.clone(), kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    q = S.qkv_headnorm_rope(y, qn, kn, 1e-6, 1, hq, hk, d, k1, v1, pos, inv_freq)
+    ref = S.attn_decode(q, k1, v1, pos + 1)
+    out = S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k2, v2, pos, inv_freq)
+    assert torch.equal(out, ref)
+    assert torch.equal(k2, k1) and torch.equal(v2, v1)
+    assert not torch.equal(k2[:, pos], kc[:, pos])                       # the row was written
+    out3 = S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k3, v3, torch.tensor([pos], device="cuda"), inv_freq)
+    assert torch.equal(out3, ref) and torch.equal(k3, k1) and torch.equal(v3, v1)
+    with pytest.raises(ValueError):
+        S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k2, v2, rows, inv_freq)
+
+
+@pytest.mark.parametrize("graphs", [False, True, "step"])
+def test_fused_attention_decoder_equals_the_two_kernel_decoder(tiny, graphs):
+    Q, args, state, packed = tiny
+    ids = torch.randint(0, args.vocab_size, (22,), generator=torch.Generator().manual_seed(8)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    c1, c2 = m.make_cache(32), m.make_cache(32)
+    m.hidden(ids[:16], c1)
+    m.hidden(ids[:16], c2)
+    two, one = Q.DecodeQwen3(m, graphs=graphs, fuse_attn=False), Q.DecodeQwen3(m, graphs=graphs, fuse_attn=True)
+    for j in range(16, 22):
+        a = two.step(ids[j:j + 1], c1).clone()
+        b = one.step(ids[j:j + 1], c2).clone()
+        torch.cuda.synchronize()
+        assert c1[0].offset == c2[0].offset == j + 1
+        assert torch.equal(a, b), j
+    assert all(torch.equal(x.k, z.k) and torch.equal(x.v, z.v) for x, z in zip(c1, c2))
+
+
 def test_packed_output_head(tiny):
     """head="packed": logits through the W4A8 GEMV on the quantized output projection, against the bf16 head."""
     Q, args, state, packed = tiny
