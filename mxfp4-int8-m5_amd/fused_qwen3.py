@@ -12,7 +12,9 @@ epilogue="row":  INT32 GEMM out, then the row kernels res_norm_quant / swiglu_qu
                  e2e/fused_qwen3.py:257-308.
 The decode step's fixed-shape halves can be captured in HIP graphs (graphs=True), which is what mx.compile does for
 the reference (e2e/decode.py:30-33): one graph launch replaces about ten kernel launches per layer."""
-from dataclasses import dataclass
+import json
+import os
+from dataclasses import dataclass, fields
 
 import torch
 import torch.nn.functional as TF
@@ -337,3 +339,77 @@ class DecodeQwen3:
             else:
                 h = self._replay(("post", i), lambda x, r, nw=nw, ws=ws: self._post(x, r, nw, ws), [o, h])
         return self._logits(h)
+
+
+# ---- from a checkpoint directory -----------------------------------------------------------------------------------
+
+def read_checkpoint(model_dir):
+    """A local Hugging Face checkpoint directory (config.json + *.safetensors) -> (Qwen3Args, state dict of CPU
+    tensors).  Nothing is fetched: the directory must hold the files."""
+    from safetensors import safe_open
+    with open(os.path.join(model_dir, "config.json")) as fh:
+        cfg = json.load(fh)
+    known = {f.name for f in fields(Qwen3Args)}
+    kw = {k: v for k, v in cfg.items() if k in known}
+    if "head_dim" not in kw:
+        kw["head_dim"] = cfg["hidden_size"] // cfg["num_attention_heads"]
+    args = Qwen3Args(**kw)
+    files = sorted(f for f in os.listdir(model_dir) if f.endswith(".safetensors"))
+    if not files:
+        raise FileNotFoundError(f"{model_dir}: no .safetensors weight files")
+    state = {}
+    for name in files:
+        with safe_open(os.path.join(model_dir, name), framework="pt", device="cpu") as fh:
+            for key in fh.keys():
+                state[key] = fh.get_tensor(key)
+    return args, state
+
+
+def load_fused(model_dir, cache_dir, resident=False, epilogue="gemm", packed="rtn"):
+    """The counterpart of e2e/fused_qwen3.py:304-338 for a checkpoint directory on disk: returns (FusedQwen3,
+    tokenizer or None).  packed="rtn": round-to-nearest SC-MXFP4 in the byte-shift cache
+    "<name>-scmxfp4.safetensors" under cache_dir (keys layers.{i}.{path}.codes / .shifts / .wscale, the file the
+    reference's pack_model writes, e2e/w4a8_mlx.py:175-195), packed on the GPU on first use; "gptq": the same format
+    from "<name>-scmxfp4-gptq.safetensors", which must exist (the GPTQ packer is not part of this library);
+    "fmt:<family member>": the cache of e2e/pack_format.py, written on first use by the device quantizer of the
+    family.  The rotated-basis caches ("rot:", "rotdown:") are not supported."""
+    from . import pack_format as PF
+    from . import sc_weights as W
+    args, state = read_checkpoint(model_dir)
+    name = os.path.basename(os.path.normpath(model_dir))
+    n_layers = args.num_hidden_layers
+    lin = lambda: {f"layers.{i}.{path}": state[f"model.layers.{i}.{path}.weight"]   # noqa: E731
+                   for i in range(n_layers) for paths in GROUPS.values() for path in paths}
+    os.makedirs(cache_dir, exist_ok=True)
+    fmt = None
+    if packed.startswith(("rot:", "rotdown:")):
+        raise NotImplementedError("weights packed in the rotated basis are not supported by this driver")
+    if packed.startswith("fmt:"):
+        member = packed[4:]
+        fmt = PF.sc_format_of(member)
+        cache = PF.cache_path(name, member, cache_dir)
+        if not os.path.exists(cache):
+            flat = {}
+            for key, w in lin().items():
+                codes, bc, ws, _ = PF.pack_matrix(w.cuda(), member, fmt)
+                flat[key + ".codes"], flat[key + ".bcodes"], flat[key + ".wscale"] = codes, bc, ws
+            W.save_cache(cache, flat)
+        pk = W.load_cache(cache)
+    elif packed in ("rtn", "gptq"):
+        cache = os.path.join(cache_dir, name + {"rtn": "-scmxfp4.safetensors", "gptq": "-scmxfp4-gptq.safetensors"}[packed])
+        if not os.path.exists(cache):
+            if packed == "gptq":
+                raise FileNotFoundError(f"{cache} is missing (written by the reference's e2e/gptq_pack.py)")
+            flat, out = pack_weights(lin()), {}
+            for key in sorted(k[:-6] for k in flat if k.endswith(".codes")):
+                c, sh, ws = F.to_shift_layout(flat[key + ".codes"], flat[key + ".bcodes"], flat[key + ".wscale"])
+                out[key + ".codes"], out[key + ".shifts"], out[key + ".wscale"] = c, sh, ws
+            W.save_cache(cache, out)
+        pk = W.load_packed(cache, n_layers)
+    else:
+        raise ValueError(f"unknown packed={packed!r}")
+    tok = None
+    if any(os.path.exists(os.path.join(model_dir, f)) for f in ("tokenizer.json", "tokenizer_config.json")):
+        from transformers import AutoTokenizer
+        tok = AutoTokenizer.from_pretrained(model_dir, local_files_only=True)
+    return FusedQwen3(args, state, pk, resident=resident, epilogue=epilogue, fmt=fmt), tok

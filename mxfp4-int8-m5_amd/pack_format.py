@@ -3,6 +3,7 @@ w[n, k] = base[n] * mult[n, k // B] * sign * code, on the device.  Mirrors the r
 (sc_format_of :35-42, pack_matrix :45-50) with the quantizer of sim/formats.py:64-107 running as a HIP kernel
 (scmx_quantize_family) instead of numpy; results are bit-identical."""
 import math
+import os
 
 import numpy as np
 import torch
@@ -22,6 +23,11 @@ CODEBOOKS = {                                   # 8 code magnitudes per codebook
 
 def slug(name):
     return name.replace("/", "_").replace(".", "")
+
+
+def cache_path(repo, name, cache_dir):
+    """File name of a model's packed cache in family member `name` (e2e/pack_format.py:79-80)."""
+    return os.path.join(cache_dir, repo.replace("/", "--") + f"-fmt-{slug(name)}.safetensors")
 
 
 def sc_format_of(name):

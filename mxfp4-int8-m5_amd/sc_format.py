@@ -89,6 +89,17 @@ def from_shift_layout(codes_u32, shifts, wscale, fmt=None):
             np.asarray(wscale, np.float32))
 
 
+def to_shift_layout(codes_u32, bcodes, wscale, fmt=None):
+    """The inverse of from_shift_layout: packed 2-bit block codes -> shifts uint8 [N, K/32] (one byte per block), the
+    layout of the round-to-nearest weight cache (e2e/w4a8_mlx.py:167-195)."""
+    fmt = fmt or DEFAULT
+    assert tuple(fmt.mult) == (1, 2, 4, 8), "the shift layout is the power-of-two format"
+    bc = np.asarray(bcodes, np.uint8)
+    parts = [(bc >> (fmt.bc_bits * j)) & ((1 << fmt.bc_bits) - 1) for j in range(fmt.per_byte)]
+    shifts = np.stack(parts, axis=-1).reshape(bc.shape[0], -1)
+    return np.asarray(codes_u32, np.uint32).reshape(-1), np.ascontiguousarray(shifts, np.uint8), np.asarray(wscale, np.float32)
+
+
 def to_device(codes, bcodes, wscale, device="cuda"):
     """numpy packed arrays -> torch tensors (codes as int32 bit patterns; torch has no uint32 arithmetic)."""
     return (torch.from_numpy(np.ascontiguousarray(codes, np.uint32).view(np.int32)).to(device),

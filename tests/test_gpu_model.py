@@ -281,6 +281,66 @@ def test_packed_output_head(tiny):
     assert int(a.argmax()) == int(b.argmax()) or rel(b, a) < 0.1
 
 
+def _write_checkpoint(path, args, state):
+    import dataclasses
+    import json
+    import os
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    cfg = dataclasses.asdict(args)
+    cfg.update(model_type="qwen3", architectures=["Qwen3ForCausalLM"])
+    with open(os.path.join(path, "config.json"), "w") as fh:
+        json.dump(cfg, fh)
+    keys = sorted(state)
+    half = len(keys) // 2   # two shards, as large checkpoints come
+    save_file({k: state[k].to(torch.bfloat16).contiguous() for k in keys[:half]}, os.path.join(path, "model-00001-of-00002.safetensors"))
+    save_file({k: state[k].to(torch.bfloat16).contiguous() for k in keys[half:]}, os.path.join(path, "model-00002-of-00002.safetensors"))
+
+
+def test_load_fused_from_a_checkpoint_directory(tiny, tmp_path):
+    """config.json + sharded safetensors on disk -> packed on the device on first use (byte-shift cache, the
+    reference's file layout), read back from the cache on the second; both equal the model quantized in memory."""
+    import os
+    from safetensors.numpy import load_file
+    Q, args, state, packed = tiny
+    ckpt, cache_dir = str(tmp_path / "tiny-qwen3"), str(tmp_path / "cache")
+    _write_checkpoint(ckpt, args, state)
+    ids = torch.randint(0, args.vocab_size, (50,), generator=torch.Generator().manual_seed(11)).cuda()
+    ref = Q.FusedQwen3(args, state, packed).hidden(ids)
+    m1, tok = Q.load_fused(ckpt, cache_dir)
+    assert tok is None and m1.args == args
+    cache = os.path.join(cache_dir, "tiny-qwen3-scmxfp4.safetensors")
+    flat = load_file(cache)
+    key = "layers.1.mlp.down_proj"
+    assert flat[key + ".shifts"].shape == (256, 512 // 32) and flat[key + ".shifts"].max() <= 3
+    assert flat[key + ".codes"].dtype == np.uint32 and flat[key + ".wscale"].dtype == np.float32
+    assert torch.equal(m1.hidden(ids), ref)
+    stamp = os.path.getmtime(cache)
+    m2, _ = Q.load_fused(ckpt, cache_dir, resident=True, epilogue="row")
+    assert os.path.getmtime(cache) == stamp                      # second use reads the cache
+    assert rel(m2.hidden(ids), ref) < 1e-2
+    with pytest.raises(FileNotFoundError):
+        Q.load_fused(ckpt, cache_dir, packed="gptq")
+    with pytest.raises(NotImplementedError):
+        Q.load_fused(ckpt, cache_dir, packed="rot:e2m1/B32/pow2")
+
+
+def test_load_fused_in_a_family_format(tiny, tmp_path):
+    import os
+    Q, args, state, packed = tiny
+    ckpt, cache_dir = str(tmp_path / "tiny-qwen3"), str(tmp_path / "cache")
+    _write_checkpoint(ckpt, args, state)
+    ids = torch.randint(0, args.vocab_size, (40,), generator=torch.Generator().manual_seed(12)).cuda()
+    member = "e2m1/B16/M1..10"
+    m, _ = Q.load_fused(ckpt, cache_dir, packed="fmt:" + member)
+    assert os.path.exists(os.path.join(cache_dir, "tiny-qwen3-fmt-e2m1_B16_M110.safetensors"))
+    assert m.fmt.block == 16 and m.fmt.bc_bits == 4
+    ref = Q.FusedQwen3(args, state, packed).hidden(ids)
+    assert rel(m.hidden(ids), ref) < 0.25                        # two different 4-bit quantizations of one model
+    m_again, _ = Q.load_fused(ckpt, cache_dir, packed="fmt:" + member)
+    assert torch.equal(m_again.hidden(ids), m.hidden(ids))
+
+
 # ---- OLMoE ---------------------------------------------------------------------------------------------------------
 
 @pytest.fixture(scope="module")

@@ -99,3 +99,38 @@ def test_mxfp4_scales_match_the_oracle_view(W):
     pw.wscale = pw.wscale * 1.5
     with pytest.raises(ValueError):
         W.mxfp4_scales(pw)
+
+
+def test_shift_layout_round_trip():
+    """to_shift_layout undoes from_shift_layout: one shift byte per 32-block <-> four 2-bit codes per byte."""
+    from mxfp4_int8_m5_amd import sc_format as F
+    rng = np.random.default_rng(3)
+    n, k = 24, 512
+    codes = rng.integers(0, 2 ** 32, n * k // 8, dtype=np.uint64).astype(np.uint32)
+    shifts = rng.integers(0, 4, (n, k // 32)).astype(np.uint8)
+    ws = (2.0 ** rng.integers(-12, -4, n)).astype(np.float32)
+    c, bc, w = F.from_shift_layout(codes, shifts, ws)
+    assert bc.shape == (n, k // 128)
+    c2, sh2, w2 = F.to_shift_layout(c, bc, w)
+    assert np.array_equal(c2, codes) and np.array_equal(sh2, shifts) and np.array_equal(w2, ws)
+    assert sh2.dtype == np.uint8 and c2.dtype == np.uint32
+
+
+def test_read_checkpoint_directory(tmp_path):
+    import json
+    import torch
+    from safetensors.torch import save_file
+    from mxfp4_int8_m5_amd import fused_qwen3 as Q
+    cfg = dict(hidden_size=64, intermediate_size=128, num_hidden_layers=1, num_attention_heads=4, num_key_value_heads=2,
+               rms_norm_eps=1e-5, rope_theta=10000.0, vocab_size=50, tie_word_embeddings=False, model_type="qwen3",
+               torch_dtype="bfloat16")
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file({"model.norm.weight": torch.ones(64), "lm_head.weight": torch.zeros(50, 64)}, str(tmp_path / "a.safetensors"))
+    save_file({"model.embed_tokens.weight": torch.zeros(50, 64)}, str(tmp_path / "b.safetensors"))
+    args, state = Q.read_checkpoint(str(tmp_path))
+    assert args.head_dim == 16 and args.rms_norm_eps == 1e-5 and args.tie_word_embeddings is False
+    assert sorted(state) == ["lm_head.weight", "model.embed_tokens.weight", "model.norm.weight"]
+    with pytest.raises(FileNotFoundError):
+        (tmp_path / "empty").mkdir()
+        (tmp_path / "empty" / "config.json").write_text(json.dumps(cfg))
+        Q.read_checkpoint(str(tmp_path / "empty"))
