@@ -292,6 +292,75 @@ def main():
         del gu, dn, x
         torch.cuda.empty_cache()
 
+        # ---- config 4: 256 routed experts + 1 shared (top-8 + shared = 9 slots), hidden 2048, intermediate 512, the
+        # 16-element-block power-of-two format; random code words (the kernels' time does not depend on the values)
+        from mxfp4_int8_m5_amd import sc_decode as SD, sc_format as SF
+        f16 = SF.Format(block=16)
+        T4, E4, D4, F4, TM4 = 2048, 257, 2048, 512, 64
+        R4 = T4 * 9
+        gen = torch.Generator(device=dev).manual_seed(4)
+
+        def experts16(n, k):
+            return (torch.randint(-2 ** 31, 2 ** 31 - 1, (E4, n * k // 8), dtype=torch.int32, device=dev, generator=gen),
+                    torch.randint(0, 256, (E4, n, k // 64), dtype=torch.uint8, device=dev, generator=gen),
+                    torch.full((E4, n), 2.0 ** -9, dtype=torch.float32, device=dev))
+        gu4, dn4 = experts16(2 * F4, D4), experts16(D4, F4)
+        lg = rng.standard_normal((T4, E4 - 1)) + rng.standard_normal(E4 - 1) * 1.5
+        top = np.argsort(-lg, axis=1)[:, :8]
+        inds4 = up(np.concatenate([top, np.full((T4, 1), E4 - 1)], 1).astype(np.int32))
+        x4 = up(acts(rng, T4, D4)).to(torch.bfloat16)
+
+        def pass4():
+            xq, xs = SK.act_quant(x4, T4)
+            pos, tok, _, off, tstart, mt = SM.route_sort(inds4, E4, TM4)
+            h = SM.moe_mm(xq, R4, gu4[0], gu4[1], gu4[2], off, tstart, mt, 2 * F4, 3, xscale=xs, tile=(TM4, 64, 4),
+                          gather=tok, fmt=f16)
+            hq, hs = SK.act_quant(h, R4)
+            return SM.moe_mm(hq, R4, dn4[0], dn4[1], dn4[2], off, tstart, mt, D4, 1, xscale=hs, tile=(TM4, 64, 4), fmt=f16)
+
+        for _ in range(3):
+            pass4()
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(20):
+            pass4()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms4 = e0.elapsed_time(e1) / 20
+        # batch-1 decode: the 9-slot gate|up and down GEMVs of one token, replayed from a HIP graph
+        xq1, xs1 = SK.act_quant(x4[:1].contiguous(), 1)
+        eidx = inds4[0, :8].contiguous()
+
+        def token4():
+            a1 = SD.gemv(xq1, gu4[0], gu4[1], xs1, gu4[2], 2 * F4, 3, eidx=eidx, xstride=0, shared=E4 - 1, fmt=f16)
+            return SD.gemv(a1, dn4[0], dn4[1], None, dn4[2], D4, 1, eidx=eidx, xstride=1, pro=1, shared=E4 - 1, fmt=f16)
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            token4()
+        stream.wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            token4()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(100):
+            graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us_tok = e0.elapsed_time(e1) / 100 * 1e3
+        bytes_tok = 9 * 3 * F4 * D4 * (0.5 + 1.0 / 64)
+        ops4 = 2.0 * R4 * 3 * F4 * D4
+        moe["config4"] = {"workload": "BASELINE configs[4]: 257 experts (256 routed + shared), 9 slots per token, 16-block "
+                                      "format; prefill of 2048 tokens (act quant, sort, two grouped GEMMs, act quant) and "
+                                      "the two 9-slot GEMVs of one decode token",
+                          "prefill_ms": round(ms4, 4), "prefill_tops": round(ops4 / ms4 / 1e9, 1), "row_tile": TM4,
+                          "decode_us_per_token": round(us_tok, 2), "decode_gbps": round(bytes_tok / us_tok / 1e3, 1)}
+        del gu4, dn4, graph
+        torch.cuda.empty_cache()
+
     # ---- decode GEMV: achieved HBM GB/s, weights rotating beyond the cache -----------------------------------------
     decode = {}
     if not a.no_decode:

@@ -34,10 +34,15 @@ struct GemmArgs {
     DevFormat fmt;
 };
 
-enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2 };
+// B_PACKED_DEFAULT / B_PACKED_B16: the published codebook with power-of-two shifts on 32- / 16-element blocks (decoded
+// with the FP4 conversion); B_PACKED_GENERIC: any member of the format family (table decode).
+enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3 };
 
 // FD = number of fragment register buffers: fragments are fetched FD - 1 k slices ahead of their MFMAs.
-template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2>
+// SKIP (grouped launches): a row tile that ends inside its expert's segment multiplies only the 32-row blocks that hold
+// valid rows.  The two waves that share a SIMD then own the same columns and different row halves of the tile, so that
+// a half-empty tile halves the MFMA work of every SIMD instead of idling two of the four.
+template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false>
 __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs a) {
     constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
     constexpr int NT = WGM * WGN * 64;
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     auto swz = [](int row, int chunk) { return row * BK + ((chunk ^ ((row / RPB) & (CPR - 1))) << 4); };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave % WGM, wn = wave / WGM;
+    const int wm = SKIP ? wave / WGN : wave % WGM, wn = SKIP ? wave % WGN : wave / WGM;
 
     // ---- which tile ------------------------------------------------------------------------------------------
     const int num_n = (a.N + BN - 1) / BN;
@@ -104,6 +109,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         row_end = a.M;
     }
     const int K = a.K;
+    // 32-row blocks of this wave's tile that hold rows of the segment (wave-uniform)
+    const int mi_active =
+        SKIP ? __builtin_amdgcn_readfirstlane(min(MI, max(0, (row_end - (m0 + wm * WTM) + 31) / 32))) : MI;
     if (a.xscale) {   // published by the barrier that opens the K loop
         for (int r = tid; r < BM; r += NT) {
             const int m = m0 + r;
@@ -150,7 +158,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             const int row = c / RUNS, kb = c % RUNS;
             const int gn = min(n0 + row, a.N - 1);
             b_src[j] = gn * (K / 2) + kb * 4 * WPC;
-            b_bc[j] = gn * a.bc_row_bytes;
+            // the block-code byte of the run: 4 blocks per byte, i.e. 128 weights (one byte per K step at most) or 64
+            b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16 ? (kb * 8 * WPC) >> 6 : 0);
             b_dst[j] = BM * BK + swz(row, kb * WPC / 2);
             b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
             b_k[j] = kb * 8 * WPC;
@@ -190,6 +199,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                     }
                     if (BMODE == B_PACKED_DEFAULT)   // 32-blocks, 2-bit codes, 4 blocks per byte: keep the raw byte
                         r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 7, 0);
+                    if (BMODE == B_PACKED_B16)       // 16-blocks: a byte covers 64 weights
+                        r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 6, 0);
                 }
             }
     };
@@ -220,6 +231,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                         if (w * NKK / WPC != q) continue;
                         if (BMODE == B_PACKED_DEFAULT) {
                             const uint32_t blk = uint32_t(k0 + b_k[j]) >> 5;
+                            decode_word_fp4(r.b[j][w], fp4_scale((uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u), o[j][2 * w],
+                                            o[j][2 * w + 1]);
+                        } else if (BMODE == B_PACKED_B16) {
+                            const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> 4;
                             decode_word_fp4(r.b[j][w], fp4_scale((uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u), o[j][2 * w],
                                             o[j][2 * w + 1]);
                         } else {
@@ -280,8 +295,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     static_assert(AHEAD >= 1 && AHEAD <= NKK, "fragment prefetch distance");
     v4i fa[FD][MI], fb[FD][NI];
     auto load_frags = [&](const int8_t* src, int kk, v4i (&xa)[MI], v4i (&xb)[NI]) {
+        if (SKIP && mi_active == 0) return;
 #pragma unroll
-        for (int i = 0; i < MI; ++i) xa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
+        for (int i = 0; i < MI; ++i)
+            if (!SKIP || i < mi_active) xa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
 #pragma unroll
         for (int j = 0; j < NI; ++j) xb[j] = *reinterpret_cast<const v4i*>(src + b_frag + j * 32 * BK + koff[kk]);
     };
@@ -308,10 +325,12 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                 load_frags(nxt, kk + AHEAD - NKK, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
             if (FD > 2) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
+            for (int i = 0; i < MI; ++i) {
+                if (SKIP && i >= mi_active) continue;
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], fa[(ph + kk) % FD][i], acc[i][j], 0, 0, 0);
+            }
             stage_slice(r, dst, k2, kk, o);
             if (FD > 2) __builtin_amdgcn_sched_barrier(0);
         }
@@ -479,7 +498,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
 
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2>
+template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false>
 static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStream_t s) {
     GemmArgs a = a_in;
     if (a.epi == SCMX_EPI_SWIGLU) a.silu = silu_table_device();
@@ -487,11 +506,17 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
     if (a.tstart) row_tiles = (row_tiles + 7) & ~7;   // grouped: whole chunks of 8 row-tile slots (spare slots exit at once)
     const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * 64);
     if (bmode == B_INT8)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD><<<grid, block, 0, s>>>(a);
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
     else if (bmode == B_PACKED_DEFAULT)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD><<<grid, block, 0, s>>>(a);
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+    else if (bmode == B_PACKED_B16)
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
     else
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD><<<grid, block, 0, s>>>(a);
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+}
+
+static int packed_mode(const DevFormat& f) {
+    return is_default_format(f) ? B_PACKED_DEFAULT : is_pow2_block16_format(f) ? B_PACKED_B16 : B_PACKED_GENERIC;
 }
 
 // Dense: the largest tile that still gives every CU a workgroup.  256x256 (wave tiles of 128x64, K steps of 64) moves
@@ -585,7 +610,7 @@ int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, 
     a.xq = xq; a.xscale = xscale; a.codes = codes; a.bcodes = bcodes; a.wscale = wscale; a.res = res; a.out = out;
     a.M = M; a.N = N; a.K = K; a.epi = epi; a.fmt = f;
     a.bc_row_bytes = K / f.block * f.bc_bits / 8;
-    launch_dense(a, is_default_format(f) ? B_PACKED_DEFAULT : B_PACKED_GENERIC, (hipStream_t)stream);
+    launch_dense(a, packed_mode(f), (hipStream_t)stream);
     return check_launch("mm_w4a8");
 }
 
@@ -633,7 +658,7 @@ static int moe_common(const char* who, const int8_t* xq, const float* xscale, co
 static void launch_grouped(const GemmArgs& a, int bmode, int tm, hipStream_t s) {
     const int max_tiles = (a.M + tm - 1) / tm + a.n_experts;   // e2e/sc_moe.py:155
     if (tm == 256 && (a.N % 256 == 0 || a.N >= 1024))   // 256-wide column tiles: fewer LDS bytes per MFMA
-        launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, max_tiles, s);
+        launch_tile<256, 256, 64, 2, 4, 1, 2, true>(a, bmode, max_tiles, s);
     else if (tm == 256)
         launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
     else if (tm == 128)
@@ -657,7 +682,7 @@ int scmx_moe_mm(const scmx_format* fmt, const int8_t* xq, const float* xscale, c
     if (R == 0) return SCMX_OK;
     a.codes = codes; a.bcodes = bcodes; a.fmt = f;
     a.bc_row_bytes = K / f.block * f.bc_bits / 8;
-    launch_grouped(a, is_default_format(f) ? B_PACKED_DEFAULT : B_PACKED_GENERIC, tm, (hipStream_t)stream);
+    launch_grouped(a, packed_mode(f), tm, (hipStream_t)stream);
     return check_launch("moe_mm");
 }
 

@@ -249,8 +249,11 @@ template <int BATCH, int R, int MODE>
 __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     constexpr int NT = 256;
     constexpr int NV = R * BATCH;
+    // MODE 0: any member of the format family (table decode); 1: published format, integer dot products; 2: published
+    // format through the FP4 conversion; 3: the same codebook and shifts on 16-element blocks through the FP4 conversion
     constexpr bool DEFAULT_FMT = MODE != 0;
-    constexpr bool FP4 = MODE == 2;
+    constexpr bool FP4 = MODE >= 2;
+    constexpr bool B16 = MODE == 3;
     constexpr int XB = FP4 ? 2 : 1;                    // bytes per staged activation
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int K = a.K, N = a.N;
@@ -295,7 +298,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             it.w[r] = __builtin_amdgcn_raw_buffer_load_b128(rc, int(16u * cc), r * (K / 2), 0);
-            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> 2), r * a.bc_row_bytes, 0);
+            // the byte with the chunk's block codes: 4 blocks per byte = 4 chunks of 32 weights, or 2 with 16-blocks
+            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> (B16 ? 1 : 2)), r * a.bc_row_bytes, 0);
         }
     };
     auto compute_item = [&](const Item& it, int g, uint32_t c_in, int (&acc)[NV]) {
@@ -306,10 +310,15 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         (void)brow;
         if constexpr (FP4) {
             float part[R][BATCH];
-            float scale[R];   // 2^(shift + 1): the codes are E2M1 values, the INT8 embedding is twice the value
+            float scale[R][2];   // 2^(shift + 1) of words 0-1 and 2-3: the codes are E2M1 values, the INT8 embedding is twice the value
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                scale[r] = __uint_as_float((128u + ((bc[r] >> (2 * (c & 3))) & 3u)) << 23);
+                if (B16) {
+                    scale[r][0] = __uint_as_float((128u + ((bc[r] >> (4 * (c & 1))) & 3u)) << 23);
+                    scale[r][1] = __uint_as_float((128u + ((bc[r] >> (4 * (c & 1) + 2)) & 3u)) << 23);
+                } else {
+                    scale[r][0] = scale[r][1] = __uint_as_float((128u + ((bc[r] >> (2 * (c & 3))) & 3u)) << 23);
+                }
 #pragma unroll
                 for (int b = 0; b < BATCH; ++b) part[r][b] = 0.0f;
             }
@@ -322,10 +331,10 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const uint32_t wj = w[r][j];
-                    const h2 q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 0);
-                    const h2 q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 1);
-                    const h2 q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 2);
-                    const h2 q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r], 3);
+                    const h2 q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r][j >> 1], 0);
+                    const h2 q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r][j >> 1], 1);
+                    const h2 q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r][j >> 1], 2);
+                    const h2 q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r][j >> 1], 3);
 #pragma unroll
                     for (int b = 0; b < BATCH; ++b) {
                         float p = part[r][b];
@@ -646,7 +655,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const GemvArgs a) {
 }
 
 template <int BATCH, int R>
-static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
+static void launch_gemv(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
     // enough workgroups to fill the chip (4 waves each), but no more than the ~24 waves per CU that can be resident:
     // waves loop
     const int groups = a.N / R;
@@ -656,14 +665,16 @@ static void launch_gemv(const GemvArgs& a, int slots, bool dflt, hipStream_t s) 
     const dim3 grid((want + rounds - 1) / rounds, slots), block(256);   // ... the same number for every wave
     // one activation row: the FP4-conversion path (activations staged as half precision) is the faster one; with
     // more rows sharing the weight stream its extra LDS reads cost more than the integer dot products
-    const int mode = !dflt ? 0 : BATCH == 1 ? 2 : 1;
-    const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (mode == 2 ? 2 : 1) + (68 + BATCH) * sizeof(float);
+    // dflt: 1 = the published format, 2 = its 16-block variant (fast path for one activation row only), 0 = other
+    const int mode = dflt == 1 ? (BATCH == 1 ? 2 : 1) : (dflt == 2 && BATCH == 1) ? 3 : 0;
+    const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (mode >= 2 ? 2 : 1) + (68 + BATCH) * sizeof(float);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024)
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
         kernel<<<grid, block, smem, s>>>(a);
     };
     if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
+    else if (mode == 3) go(gemv_kernel<BATCH, R, 3>);
     else if (mode == 1) go(gemv_kernel<BATCH, R, 1>);
     else go(gemv_kernel<BATCH, R, 0>);
 }
@@ -682,8 +693,8 @@ static void launch_gemv_mfma(const GemvArgs& a, hipStream_t s) {
 }
 
 template <int BATCH>
-static void launch_gemv_rows(const GemvArgs& a, int slots, bool dflt, hipStream_t s) {
-    if (BATCH > 1 && dflt && !a.eidx && a.N % 4 == 0 && a.K % 512 == 0)
+static void launch_gemv_rows(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
+    if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 4 == 0 && a.K % 512 == 0)
         return launch_gemv_mfma<BATCH>(a, s);
     // more rows per wave = more loads in flight per lane; fewer = more waves for narrow layers
     const long rows = long(a.N) * slots;
@@ -744,7 +755,7 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
     a.bc_row_bytes = K / f.block * f.bc_bits / 8;
     a.eidx = eidx; a.n_eidx = n_eidx; a.xstride = xstride; a.shared_expert = eidx ? shared_expert : -1;
     a.fmt = f;
-    const bool dflt = is_default_format(f);
+    const int dflt = is_default_format(f) ? 1 : is_pow2_block16_format(f) ? 2 : 0;
     hipStream_t s = (hipStream_t)stream;
     switch (batch) {
         case 1: launch_gemv_rows<1>(a, slots, dflt, s); break;

@@ -32,6 +32,10 @@ int make_dev_format(const scmx_format* f, DevFormat* out);
 inline bool is_default_format(const DevFormat& d) {
     return d.lut_lo == 0x03020100u && d.lut_hi == 0x0C080604u && d.block == 32 && d.bc_bits == 2 && d.pow2;
 }
+// The same codebook and power-of-two shifts on 16-element blocks (one 2-bit code per two code words).
+inline bool is_pow2_block16_format(const DevFormat& d) {
+    return d.lut_lo == 0x03020100u && d.lut_hi == 0x0C080604u && d.block == 16 && d.bc_bits == 2 && d.pow2;
+}
 
 // Thread-local error text behind scmx_last_error().
 void set_error(const char* fmt, ...);

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import bf16, layout, linear
-from tests.util import FORMATS, dev, host, product_format, random_packed
+from tests.util import FORMATS, dev, host, llm_acts, product_format, random_packed
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -57,6 +57,33 @@ def test_gemv_formats(G, i):
     xs = np.array([1e-2], F32)
     y = host(G.gemv(dev(xq), dev(codes), dev(bc), dev(xs), dev(ws), n, 1, fmt=product_format(fmt)))
     assert np.array_equal(y, linear.gemv(xq, xs[0], q, ws, 1))
+
+
+@pytest.mark.parametrize("n,k", [(512, 6144), (64, 1024), (20, 128), (1024, 2048)])
+def test_gemv_block16_power_of_two_format(G, n, k):
+    """The 16-element-block variant of the published format (its own conversion path in the kernel): saturated
+    activations, every epilogue, rows that take several passes over K, and a fused act_quant prologue."""
+    fmt = layout.Format(block=16)
+    pf = product_format(fmt)
+    rng = np.random.default_rng(n + k + 16)
+    codes, bc, ws, q = random_packed(rng, n, k, fmt)
+    xq = rng.integers(-127, 128, k).astype(np.int8)
+    xq[:16] = 127
+    xs = np.array([0.01], F32)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    ref1 = linear.gemv(xq, xs[0], q, ws, 1)
+    assert np.array_equal(host(G.gemv(dev(xq), dc, db, dev(xs), dw, n, 1, fmt=pf)), ref1)
+    res = bf16.to_bits(rng.standard_normal(n).astype(F32))
+    y2 = host(G.gemv(dev(xq), dc, db, dev(xs), dw, n, 2, res=dev(res), fmt=pf))
+    assert np.array_equal(y2, linear.gemv(xq, xs[0], q, ws, 2, res))
+    perm = linear.interleave_gate_up(n // 2)
+    cp = codes.reshape(n, -1)[perm].reshape(-1)
+    y3 = host(G.gemv(dev(xq), dev(cp), dev(bc[perm]), dev(xs), dev(ws[perm]), n, 3, fmt=pf))
+    assert np.array_equal(y3, linear.swiglu(ref1[:n // 2], ref1[n // 2:]))
+    xb, x = llm_acts(rng, 1, k)
+    rq, rs = linear.act_quant(x)
+    yp = host(G.gemv(dev(xb), dc, db, None, dw, n, 1, pro=1, fmt=pf))
+    assert np.array_equal(yp, linear.gemv(rq[0], rs[0], q, ws, 1))
 
 
 @pytest.mark.parametrize("pro", [1, 2])

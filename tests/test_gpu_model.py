@@ -9,6 +9,15 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def default_format_afterwards():
+    """The model drivers select their weight format globally (as the reference's set_format does); leave the default
+    behind for whatever runs next."""
+    yield
+    from mxfp4_int8_m5_amd import sc_format, sc_kernels
+    sc_kernels.set_format(sc_format.Format())
+
+
 @pytest.fixture(scope="module")
 def tiny():
     from mxfp4_int8_m5_amd import fused_qwen3 as Q, sc_weights as W
