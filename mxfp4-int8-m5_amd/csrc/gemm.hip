@@ -35,8 +35,10 @@ struct GemmArgs {
 };
 
 // B_PACKED_DEFAULT / B_PACKED_B16: the published codebook with power-of-two shifts on 32- / 16-element blocks (decoded
-// with the FP4 conversion); B_PACKED_GENERIC: any member of the format family (table decode).
-enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3 };
+// with the FP4 conversion); B_PACKED_B16M: that codebook on 16-element blocks with 4-bit codes for consecutive integer
+// multipliers (FP4 conversion, then one fused multiply-add); B_PACKED_GENERIC: any member of the format family (table
+// decode).
+enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3, B_PACKED_B16M = 4 };
 
 // FD = number of fragment register buffers: fragments are fetched FD - 1 k slices ahead of their MFMAs.
 // SKIP (grouped launches): a row tile that ends inside its expert's segment multiplies only the 32-row blocks that hold
@@ -159,7 +161,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             const int gn = min(n0 + row, a.N - 1);
             b_src[j] = gn * (K / 2) + kb * 4 * WPC;
             // the block-code byte of the run: 4 blocks per byte, i.e. 128 weights (one byte per K step at most) or 64
-            b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16 ? (kb * 8 * WPC) >> 6 : 0);
+            // (two 4-bit codes per byte: 32)
+            b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16    ? (kb * 8 * WPC) >> 6
+                                             : BMODE == B_PACKED_B16M ? (kb * 8 * WPC) >> 5
+                                                                      : 0);
             b_dst[j] = BM * BK + swz(row, kb * WPC / 2);
             b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
             b_k[j] = kb * 8 * WPC;
@@ -201,6 +206,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                         r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 7, 0);
                     if (BMODE == B_PACKED_B16)       // 16-blocks: a byte covers 64 weights
                         r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 6, 0);
+                    if (BMODE == B_PACKED_B16M)      // 16-blocks, 4-bit codes: 32 weights
+                        r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 5, 0);
                 }
             }
     };
@@ -237,6 +244,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                             const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> 4;
                             decode_word_fp4(r.b[j][w], fp4_scale((uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u), o[j][2 * w],
                                             o[j][2 * w + 1]);
+                        } else if (BMODE == B_PACKED_B16M) {
+                            const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> 4;
+                            const _Float16 m = _Float16(int(((uint32_t(r.bc[j]) >> (4 * (blk & 1))) & 15u) + (a.fmt.mult[0] & 0xFFu)));
+                            decode_word_fp4_mul(r.b[j][w], half2_t{m, m}, o[j][2 * w], o[j][2 * w + 1]);
                         } else {
                             const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> a.fmt.block_log2;
                             const uint32_t bc = block_code(a.bcodes + erow * a.bc_row_bytes + b_bc[j], blk, a.fmt.bc_bits);
@@ -511,12 +522,17 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
         gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
     else if (bmode == B_PACKED_B16)
         gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+    else if (bmode == B_PACKED_B16M)
+        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
     else
         gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
 }
 
 static int packed_mode(const DevFormat& f) {
-    return is_default_format(f) ? B_PACKED_DEFAULT : is_pow2_block16_format(f) ? B_PACKED_B16 : B_PACKED_GENERIC;
+    return is_default_format(f)        ? B_PACKED_DEFAULT
+           : is_pow2_block16_format(f) ? B_PACKED_B16
+           : is_block16_range_format(f) ? B_PACKED_B16M
+                                        : B_PACKED_GENERIC;
 }
 
 // Dense: the largest tile that still gives every CU a workgroup.  256x256 (wave tiles of 128x64, K steps of 64) moves

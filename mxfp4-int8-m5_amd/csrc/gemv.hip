@@ -252,8 +252,10 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     // MODE 0: any member of the format family (table decode); 1: published format, integer dot products; 2: published
     // format through the FP4 conversion; 3: the same codebook and shifts on 16-element blocks through the FP4 conversion
     constexpr bool DEFAULT_FMT = MODE != 0;
+    // conversion; 4: that codebook on 16-element blocks with 4-bit codes for consecutive integer multipliers
     constexpr bool FP4 = MODE >= 2;
     constexpr bool B16 = MODE == 3;
+    constexpr bool B16M = MODE == 4;
     constexpr int XB = FP4 ? 2 : 1;                    // bytes per staged activation
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int K = a.K, N = a.N;
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         for (int r = 0; r < R; ++r) {
             it.w[r] = __builtin_amdgcn_raw_buffer_load_b128(rc, int(16u * cc), r * (K / 2), 0);
             // the byte with the chunk's block codes: 4 blocks per byte = 4 chunks of 32 weights, or 2 with 16-blocks
-            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> (B16 ? 1 : 2)), r * a.bc_row_bytes, 0);
+            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> (B16M ? 0 : B16 ? 1 : 2)), r * a.bc_row_bytes, 0);
         }
     };
     auto compute_item = [&](const Item& it, int g, uint32_t c_in, int (&acc)[NV]) {
@@ -310,10 +312,15 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         (void)brow;
         if constexpr (FP4) {
             float part[R][BATCH];
+            float part2[B16M ? R : 1][BATCH];   // integer multipliers: words 2-3 (the chunk's second block) summed apart
             float scale[R][2];   // 2^(shift + 1) of words 0-1 and 2-3: the codes are E2M1 values, the INT8 embedding is twice the value
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                if (B16) {
+                if (B16M) {
+                    scale[r][0] = scale[r][1] = 2.0f;
+#pragma unroll
+                    for (int b = 0; b < BATCH; ++b) part2[r][b] = 0.0f;
+                } else if (B16) {
                     scale[r][0] = __uint_as_float((128u + ((bc[r] >> (4 * (c & 1))) & 3u)) << 23);
                     scale[r][1] = __uint_as_float((128u + ((bc[r] >> (4 * (c & 1) + 2)) & 3u)) << 23);
                 } else {
@@ -337,19 +344,28 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
                     const h2 q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wj, scale[r][j >> 1], 3);
 #pragma unroll
                     for (int b = 0; b < BATCH; ++b) {
-                        float p = part[r][b];
+                        float& dst = (B16M && j >= 2) ? part2[B16M ? r : 0][b] : part[r][b];
+                        float p = dst;
                         p = __builtin_amdgcn_fdot2(q0, __builtin_shufflevector(xv[b], xv[b], 0, 1), p, false);
                         p = __builtin_amdgcn_fdot2(q1, __builtin_shufflevector(xv[b], xv[b], 2, 3), p, false);
                         p = __builtin_amdgcn_fdot2(q2, __builtin_shufflevector(xv[b], xv[b], 4, 5), p, false);
                         p = __builtin_amdgcn_fdot2(q3, __builtin_shufflevector(xv[b], xv[b], 6, 7), p, false);
-                        part[r][b] = p;
+                        dst = p;
                     }
                 }
             }
 #pragma unroll
-            for (int r = 0; r < R; ++r)
+            for (int r = 0; r < R; ++r) {
+                const int m0 = int(a.fmt.mult[0] & 0xFFu);
+                const int mlo = m0 + int(bc[r] & 15u), mhi = m0 + int((bc[r] >> 4) & 15u);
 #pragma unroll
-                for (int b = 0; b < BATCH; ++b) acc[r * BATCH + b] += int(part[r][b]);
+                for (int b = 0; b < BATCH; ++b) {
+                    if (B16M)
+                        acc[r * BATCH + b] += int(part[r][b]) * mlo + int(part2[r][b]) * mhi;
+                    else
+                        acc[r * BATCH + b] += int(part[r][b]);
+                }
+            }
             return;
         }
             u32x4 xv[BATCH][2];
@@ -666,7 +682,8 @@ static void launch_gemv(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
     // one activation row: the FP4-conversion path (activations staged as half precision) is the faster one; with
     // more rows sharing the weight stream its extra LDS reads cost more than the integer dot products
     // dflt: 1 = the published format, 2 = its 16-block variant (fast path for one activation row only), 0 = other
-    const int mode = dflt == 1 ? (BATCH == 1 ? 2 : 1) : (dflt == 2 && BATCH == 1) ? 3 : 0;
+    // 3 = the 16-block family members with consecutive integer multipliers (likewise)
+    const int mode = dflt == 1 ? (BATCH == 1 ? 2 : 1) : (dflt >= 2 && BATCH == 1) ? dflt + 1 : 0;
     const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (mode >= 2 ? 2 : 1) + (68 + BATCH) * sizeof(float);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024)
@@ -675,6 +692,7 @@ static void launch_gemv(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
     };
     if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
     else if (mode == 3) go(gemv_kernel<BATCH, R, 3>);
+    else if (mode == 4) go(gemv_kernel<BATCH, R, 4>);
     else if (mode == 1) go(gemv_kernel<BATCH, R, 1>);
     else go(gemv_kernel<BATCH, R, 0>);
 }
@@ -755,7 +773,7 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
     a.bc_row_bytes = K / f.block * f.bc_bits / 8;
     a.eidx = eidx; a.n_eidx = n_eidx; a.xstride = xstride; a.shared_expert = eidx ? shared_expert : -1;
     a.fmt = f;
-    const int dflt = is_default_format(f) ? 1 : is_pow2_block16_format(f) ? 2 : 0;
+    const int dflt = is_default_format(f) ? 1 : is_pow2_block16_format(f) ? 2 : is_block16_range_format(f) ? 3 : 0;
     hipStream_t s = (hipStream_t)stream;
     switch (batch) {
         case 1: launch_gemv_rows<1>(a, slots, dflt, s); break;

@@ -37,6 +37,21 @@ inline bool is_pow2_block16_format(const DevFormat& d) {
     return d.lut_lo == 0x03020100u && d.lut_hi == 0x0C080604u && d.block == 16 && d.bc_bits == 2 && d.pow2;
 }
 
+// The same codebook on 16-element blocks with 4-bit block codes whose multipliers are consecutive integers
+// (mult[i] = mult[0] + i, unused entries 0): the "B16/M<lo>..<hi>" members of the family.  A block's multiplier is then
+// its code plus mult[0], no table needed.
+inline bool is_block16_range_format(const DevFormat& d) {
+    if (!(d.lut_lo == 0x03020100u && d.lut_hi == 0x0C080604u && d.block == 16 && d.bc_bits == 4) || d.pow2) return false;
+    const uint32_t m0 = d.mult[0] & 0xFFu;
+    bool ended = false;
+    for (uint32_t i = 0; i < 16; ++i) {
+        const uint32_t m = (d.mult[i >> 2] >> (8 * (i & 3))) & 0xFFu;
+        if (m == 0) ended = true;
+        else if (ended || m != m0 + i) return false;
+    }
+    return m0 >= 1;
+}
+
 // Thread-local error text behind scmx_last_error().
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
@@ -156,6 +171,17 @@ __device__ __forceinline__ void decode_word_fp4(uint32_t w, float scale, uint32_
     const half2_t q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 1) + bias;
     const half2_t q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 2) + bias;
     const half2_t q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 3) + bias;
+    a = perm(__builtin_bit_cast(uint32_t, q1), __builtin_bit_cast(uint32_t, q0), 0x06040200u);
+    b = perm(__builtin_bit_cast(uint32_t, q3), __builtin_bit_cast(uint32_t, q2), 0x06040200u);
+}
+
+// The same with an integer multiplier per call (m = the multiplier in both halves): code value x multiplier.
+__device__ __forceinline__ void decode_word_fp4_mul(uint32_t w, half2_t m, uint32_t& a, uint32_t& b) {
+    const half2_t bias = half2_t{_Float16(1536.0f), _Float16(1536.0f)};
+    const half2_t q0 = __builtin_elementwise_fma(half2_t(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 0)), m, bias);
+    const half2_t q1 = __builtin_elementwise_fma(half2_t(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 1)), m, bias);
+    const half2_t q2 = __builtin_elementwise_fma(half2_t(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 2)), m, bias);
+    const half2_t q3 = __builtin_elementwise_fma(half2_t(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 3)), m, bias);
     a = perm(__builtin_bit_cast(uint32_t, q1), __builtin_bit_cast(uint32_t, q0), 0x06040200u);
     b = perm(__builtin_bit_cast(uint32_t, q3), __builtin_bit_cast(uint32_t, q2), 0x06040200u);
 }

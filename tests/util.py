@@ -58,4 +58,5 @@ def product_format(fmt):
 
 FORMATS = [layout.Format(), layout.Format(block=16), layout.Format(block=32, mult=(1, 2, 3, 4)),
            layout.Format(block=16, mult=(1, 2, 3, 4, 5, 6, 8, 10), bc_bits=4),
-           layout.Format(block=32, code_mag=(0, 1, 2, 3, 4, 5, 6, 7), mult=(1, 3, 9, 15))]
+           layout.Format(block=32, code_mag=(0, 1, 2, 3, 4, 5, 6, 7), mult=(1, 3, 9, 15)),
+           layout.Format(block=16, mult=tuple(range(1, 11)), bc_bits=4)]     # "e2m1/B16/M1..10": consecutive multipliers
