@@ -113,7 +113,8 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
                       int L, int hq, int hk, int d, void* stream);
 
 /* scmx_qkv_headnorm followed by the rotary embedding of q and k (pairs (i, i + d/2) of a head, angle = position *
- * inv_freq[i], inv_freq f32 [d/2]) and the append to the KV cache: q -> [hq, L, d]; k, v -> rows pos..pos+L-1 of
+ * inv_freq[i], inv_freq f32 [d/2]) and the append to the KV cache: q -> [hq, L, d] (q_token_major != 0: [L, hq, d],
+ * the layout from which an attention output needs no transpose before the o projection); k, v -> rows pos..pos+L-1 of
  * caches [hk, cache_rows, d].  pos = *pos_dev when pos_dev != NULL (a device-resident position, so that a captured
  * graph can be replayed for every token), else pos0.  With pos_dev the caller guarantees *pos_dev + L <= cache_rows.
  * Fuses what the model integrations do with array ops after qkv_headnorm_y: at.rope(q), at.rope(k),
@@ -121,7 +122,7 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
 int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
                            const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* kcache,
                            uint16_t* vcache, int L, int hq, int hk, int d, const float* inv_freq,
-                           const int64_t* pos_dev, int64_t pos0, int cache_rows, void* stream);
+                           const int64_t* pos_dev, int64_t pos0, int cache_rows, int q_token_major, void* stream);
 
 /* Single-token attention against a KV cache: out bf16 [hq * d] = softmax(q . K^T * scale) V per query head, q bf16
  * [hq, d], caches bf16 [hk, cache_rows, d] of which the first n rows are valid; n = *pos_dev + 1 when pos_dev != NULL

@@ -181,6 +181,7 @@ struct RopeArgs {
     const int64_t* pos_dev;  // optional device-resident position of row 0 (read when non-NULL), else pos0
     int64_t pos0;
     int kv_rows;             // rows per head of the k / v destinations
+    int q_token_major;       // q as [L, hq, d] instead of [hq, L, d]
 };
 
 __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
@@ -199,28 +200,42 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
         for (int i = threadIdx.x; i < d / 2; i += NT) sincosf(float(pos) * rope.inv_freq[i], &s_sin[i], &s_cos[i]);
         __syncthreads();
     }
-    // blockIdx.y strides over groups of NT / 64 heads (one per wave): a single row still fills many CUs
-    for (int g = blockIdx.y * (NT / 64) + wave; g < heads; g += gridDim.y * (NT / 64)) {
-        float yv[8];   // per <= 8 (d <= 512)
-        float ss = 0.0f;
-        for (int i = 0; i < per; ++i) {
-            const int c = g * d + per * lane + i;
-            if (acc)
-                yv[i] = round_bf16(__fmul_rn(__fmul_rn(float(acc[size_t(row) * ntot + c]), xscale[row]), wscale[c]));
-            else
-                yv[i] = bf16_to_f32(y[size_t(row) * ntot + c]);
-            ss = __fadd_rn(ss, __fmul_rn(yv[i], yv[i]));
+    // blockIdx.y strides over groups of NT / 64 heads (one per wave): a single row still fills many CUs.  A wave takes
+    // its heads U at a time with all their loads issued first, so one memory latency covers U heads.
+    constexpr int U = 4;
+    const int stride = gridDim.y * (NT / 64);
+    for (int g0 = blockIdx.y * (NT / 64) + wave; g0 < heads; g0 += U * stride) {
+        float yv[U][8];   // per <= 8 (d <= 512)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int g = g0 + u * stride;
+            if (g >= heads) break;
+            for (int i = 0; i < per; ++i) {
+                const int c = g * d + per * lane + i;
+                if (acc)
+                    yv[u][i] = round_bf16(__fmul_rn(__fmul_rn(float(acc[size_t(row) * ntot + c]), xscale[row]), wscale[c]));
+                else
+                    yv[u][i] = bf16_to_f32(y[size_t(row) * ntot + c]);
+            }
         }
-        uint16_t* out;
-        int hh;
-        if (g < hq) { out = q; hh = g; } else if (g < hq + hk) { out = k; hh = g - hq; } else { out = v; hh = g - hq - hk; }
-        uint16_t* o = g < hq ? out + (size_t(hh) * L + row) * d + per * lane
-                             : out + (size_t(hh) * kv_rows + size_t(pos)) * d + per * lane;
-        if (g < hq + hk) {
-            head_norm_rope(yv, ss, per, lane, d, g < hq ? qn : kn, eps, rope.inv_freq ? s_sin : nullptr, s_cos,
-                           [&](int i, uint16_t b) { o[i] = b; });
-        } else {
-            for (int i = 0; i < per; ++i) o[i] = f32_to_bf16(yv[i]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int g = g0 + u * stride;
+            if (g >= heads) break;
+            float ss = 0.0f;
+            for (int i = 0; i < per; ++i) ss = __fadd_rn(ss, __fmul_rn(yv[u][i], yv[u][i]));
+            uint16_t* out;
+            int hh;
+            if (g < hq) { out = q; hh = g; } else if (g < hq + hk) { out = k; hh = g - hq; } else { out = v; hh = g - hq - hk; }
+            uint16_t* o = g >= hq              ? out + (size_t(hh) * kv_rows + size_t(pos)) * d + per * lane
+                          : rope.q_token_major ? out + (size_t(row) * hq + hh) * d + per * lane
+                                               : out + (size_t(hh) * L + row) * d + per * lane;
+            if (g < hq + hk) {
+                head_norm_rope(yv[u], ss, per, lane, d, g < hq ? qn : kn, eps, rope.inv_freq ? s_sin : nullptr, s_cos,
+                               [&](int i, uint16_t b) { o[i] = b; });
+            } else {
+                for (int i = 0; i < per; ++i) o[i] = f32_to_bf16(yv[u][i]);
+            }
         }
     }
 }
@@ -504,14 +519,14 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
     }
     if (L == 0) return SCMX_OK;
     qkv_headnorm_kernel<<<headnorm_grid(L, hq + 2 * hk), dim3(NT), 0, (hipStream_t)stream>>>(
-        acc, xscale, wscale, y, qn, kn, eps, q, k, v, L, hq, hk, d, RopeArgs{nullptr, nullptr, 0, 0});
+        acc, xscale, wscale, y, qn, kn, eps, q, k, v, L, hq, hk, d, RopeArgs{nullptr, nullptr, 0, 0, 0});
     return check_launch("qkv_headnorm");
 }
 
 int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
                            const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* kcache,
                            uint16_t* vcache, int L, int hq, int hk, int d, const float* inv_freq,
-                           const int64_t* pos_dev, int64_t pos0, int cache_rows, void* stream) {
+                           const int64_t* pos_dev, int64_t pos0, int cache_rows, int q_token_major, void* stream) {
     if ((!acc && !y) || (acc && (!xscale || !wscale)) || !qn || !kn || !q || !kcache || !vcache || !inv_freq) {
         set_error("qkv_headnorm_rope: null pointer argument");
         return SCMX_ERR_ARG;
@@ -527,7 +542,7 @@ int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float*
     }
     if (L == 0) return SCMX_OK;
     qkv_headnorm_kernel<<<headnorm_grid(L, hq + 2 * hk), dim3(NT), 0, (hipStream_t)stream>>>(
-        acc, xscale, wscale, y, qn, kn, eps, q, kcache, vcache, L, hq, hk, d, RopeArgs{inv_freq, pos_dev, pos0, cache_rows});
+        acc, xscale, wscale, y, qn, kn, eps, q, kcache, vcache, L, hq, hk, d, RopeArgs{inv_freq, pos_dev, pos0, cache_rows, q_token_major});
     return check_launch("qkv_headnorm_rope");
 }
 

@@ -113,7 +113,7 @@ class FusedQwen3:
         a = self.args
         return S.qkv_headnorm_rope(y, nw["self_attn.q_norm"], nw["self_attn.k_norm"], self.eps, L, a.num_attention_heads,
                                    a.num_key_value_heads, a.head_dim, c.k, c.v, c.offset if pos is None else pos,
-                                   self.inv_freq, acc=acc, xscale=xs, wscale=ws)
+                                   self.inv_freq, acc=acc, xscale=xs, wscale=ws, token_major=L > 1)
 
     def _attend(self, c, q, L):
         """q [hq, L, d] (already rotated) against the cache, whose rows offset..offset+L-1 were just written."""
@@ -134,6 +134,8 @@ class FusedQwen3:
             pos = torch.arange(off, off + L, device=q.device)[:, None]
             mask = torch.arange(off + L, device=q.device)[None] <= pos
             o = TF.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask, **gqa)
+        # q arrives as the [hq, L, d] view of [L, hq, d] storage and the attention op lays its output out like q, so
+        # this is a view; contiguous() copies only if a backend chose another layout
         return o[0].transpose(0, 1).reshape(L, -1).contiguous()
 
     def _embed(self, ids):

@@ -228,20 +228,23 @@ def qkv_headnorm_y(y, qn, kn, eps, L, hq, hk, d, deps=()):
     return _headnorm(None, None, None, y, qn, kn, eps, L, hq, hk, d, y.device)
 
 
-def qkv_headnorm_rope(y, qn, kn, eps, L, hq, hk, d, kcache, vcache, pos, inv_freq, acc=None, xscale=None, wscale=None):
+def qkv_headnorm_rope(y, qn, kn, eps, L, hq, hk, d, kcache, vcache, pos, inv_freq, acc=None, xscale=None, wscale=None,
+                      token_major=False):
     """qkv_headnorm_y (or, with acc / xscale / wscale, qkv_epilogue_headnorm) fused with the rotary embedding of q
     and k and the KV-cache append: returns q [hq, L, d]; k and v go to rows pos..pos+L-1 of kcache / vcache
-    [hk, rows, d].  pos: int, or an int64 device tensor (for graph replay)."""
+    [hk, rows, d].  pos: int, or an int64 device tensor (for graph replay).  token_major=True stores q as [L, hq, d]
+    and returns the [hq, L, d] view of it: an attention output that inherits this layout is [L, hq * d] without a
+    transposing copy."""
     src = y if y is not None else acc
-    q = torch.empty((hq, L, d), dtype=torch.bfloat16, device=src.device)
+    q = torch.empty((L, hq, d) if token_major else (hq, L, d), dtype=torch.bfloat16, device=src.device)
     assert kcache.shape == vcache.shape and kcache.shape[0] == hk and kcache.shape[2] == d
     assert kcache.dtype == torch.bfloat16 and inv_freq.dtype == torch.float32 and inv_freq.numel() == d // 2
     dev_pos = pos if torch.is_tensor(pos) else None
     assert dev_pos is None or dev_pos.dtype == torch.int64
     _lib.call("scmx_qkv_headnorm_rope", _lib.ptr(acc), _lib.ptr(xscale), _lib.ptr(wscale), _lib.ptr(y), _lib.ptr(qn),
               _lib.ptr(kn), _eps(eps), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache), L, hq, hk, d, _lib.ptr(inv_freq),
-              _lib.ptr(dev_pos), 0 if dev_pos is not None else int(pos), kcache.shape[1], _lib.stream())
-    return q
+              _lib.ptr(dev_pos), 0 if dev_pos is not None else int(pos), kcache.shape[1], int(token_major), _lib.stream())
+    return q.transpose(0, 1) if token_major else q
 
 
 def attn_decode(q, kcache, vcache, n, scale=None):

@@ -205,6 +205,8 @@ def test_fused_headnorm_rope_append_against_separate_ops(L, pos, from_acc):
     for c in (kc, vc):
         assert bool((c[:, :pos] == 7).all()) and bool((c[:, pos + L:] == 7).all())
     kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    qt = S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc.clone(), vc.clone(), pos, inv_freq, token_major=True, **kw)
+    assert qt.shape == q.shape and torch.equal(qt, q) and qt.transpose(0, 1).is_contiguous()    # same values, [L, hq, d] storage
     q2 = S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc2, vc2, torch.tensor([pos], device="cuda"), inv_freq, **kw)
     assert torch.equal(q2, q) and torch.equal(kc2[:, pos:pos + L], kc[:, pos:pos + L])
     with pytest.raises(ValueError):
