@@ -141,6 +141,14 @@ int scmx_attn_decode_qkv(const uint16_t* y, const uint16_t* qn, const uint16_t* 
                          const int64_t* pos_dev, int64_t pos0, uint16_t* kcache, uint16_t* vcache, uint16_t* out,
                          int hq, int hk, int d, int cache_rows, float scale, void* stream);
 
+/* Causal attention of L new tokens against a KV cache that holds `off` earlier rows followed by the L new ones:
+ * q bf16 [L, hq, d] (token-major, as scmx_qkv_headnorm_rope writes it with q_token_major), caches bf16
+ * [hk, cache_rows, d], out bf16 [L, hq * d]; query i attends to cache rows 0 .. off + i.  d = 128.  float32
+ * accumulation, bf16 probabilities.  Takes the place of the array library's scaled-dot-product attention in the
+ * prefill (e2e/fused_qwen3.py:216-222); no counterpart among the reference's own kernels. */
+int scmx_attn_prefill(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, uint16_t* out, int L, int off,
+                      int hq, int hk, int d, int cache_rows, float scale, void* stream);
+
 /* OLMoE q/k/v split with RMSNorm over the full h*d width.  Replaces qkv_fullnorm_y, e2e/sc_kernels.py:390-423,
  * 629-637. */
 int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q,

@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libscmx.so")
-SOURCES = ["api.hip", "gemm.hip", "gemv.hip", "rowops.hip", "quantize.hip", "attn.hip", "silu_table.hip"]
+SOURCES = ["api.hip", "gemm.hip", "gemv.hip", "rowops.hip", "quantize.hip", "attn.hip", "attn_prefill.hip", "silu_table.hip"]
 # packed FP32 instructions are kept off (they have misbehaved on this hardware pool); no FMA contraction, so the
 # FP32 epilogues and norms round exactly like a plain IEEE evaluation
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-Wno-unused-command-line-argument", "-fconstexpr-steps=400000000",

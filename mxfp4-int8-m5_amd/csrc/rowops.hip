@@ -210,6 +210,12 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
         for (int u = 0; u < U; ++u) {
             const int g = g0 + u * stride;
             if (g >= heads) break;
+            if (!acc && per == 2) {   // head dim 128: the lane's two values in one 32-bit load
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(y + size_t(row) * ntot + g * d + 2 * lane);
+                yv[u][0] = __uint_as_float(w << 16);
+                yv[u][1] = __uint_as_float(w & 0xFFFF0000u);
+                continue;
+            }
             for (int i = 0; i < per; ++i) {
                 const int c = g * d + per * lane + i;
                 if (acc)
@@ -230,11 +236,16 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
             uint16_t* o = g >= hq              ? out + (size_t(hh) * kv_rows + size_t(pos)) * d + per * lane
                           : rope.q_token_major ? out + (size_t(row) * hq + hh) * d + per * lane
                                                : out + (size_t(hh) * L + row) * d + per * lane;
+            uint32_t pair = 0;   // per == 2: both results leave in one 32-bit store
+            auto emit = [&](int i, uint16_t b) {
+                if (per != 2) { o[i] = b; return; }
+                pair |= uint32_t(b) << (16 * i);
+                if (i == 1) *reinterpret_cast<uint32_t*>(o) = pair;
+            };
             if (g < hq + hk) {
-                head_norm_rope(yv[u], ss, per, lane, d, g < hq ? qn : kn, eps, rope.inv_freq ? s_sin : nullptr, s_cos,
-                               [&](int i, uint16_t b) { o[i] = b; });
+                head_norm_rope(yv[u], ss, per, lane, d, g < hq ? qn : kn, eps, rope.inv_freq ? s_sin : nullptr, s_cos, emit);
             } else {
-                for (int i = 0; i < per; ++i) o[i] = f32_to_bf16(yv[u][i]);
+                for (int i = 0; i < per; ++i) emit(i, f32_to_bf16(yv[u][i]));
             }
         }
     }

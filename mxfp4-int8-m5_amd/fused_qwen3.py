@@ -88,6 +88,7 @@ class FusedQwen3:
                                   device) for g, paths in GROUPS.items()}
             self.layers.append((norms, ws))
         self.sdpa_gqa = True    # let the attention op share KV heads between query heads instead of copying them
+        self.attn_kernel = True  # prefill attention through scmx_attn_prefill where it applies, else torch's op
         half = args.head_dim // 2
         self.inv_freq = 1.0 / (args.rope_theta ** (torch.arange(half, device=device, dtype=torch.float32) / half))
 
@@ -125,6 +126,8 @@ class FusedQwen3:
         hq, hk = q.shape[0], k.shape[0]
         if L == 1:
             return S.attn_decode(q, c.k, c.v, off + 1)
+        if self.attn_kernel and q.shape[-1] == 128:   # this library's causal attention (head dim 128 only)
+            return S.attn_prefill(q, c.k, c.v, off)
         gqa = {"enable_gqa": True} if hq != hk and self.sdpa_gqa else {}
         if hq != hk and not self.sdpa_gqa:
             k, v = k.repeat_interleave(hq // hk, 0), v.repeat_interleave(hq // hk, 0)

@@ -260,6 +260,20 @@ def attn_decode(q, kcache, vcache, n, scale=None):
     return out
 
 
+def attn_prefill(q, kcache, vcache, off, scale=None):
+    """Causal attention of L new tokens: q bf16 [hq, L, d], best as the view of [L, hq, d] storage that
+    qkv_headnorm_rope returns with token_major=True (any other layout is copied into that one), caches [hk, rows, d]
+    whose rows off .. off+L-1 hold the new tokens' keys and values -> bf16 [L, hq * d].  Head dim 128."""
+    q = q.transpose(0, 1).contiguous()   # [L, hq, d] storage; no copy when q already is a view of it
+    L, hq, d = q.shape
+    hk, rows, _ = kcache.shape
+    assert q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and kcache.shape == vcache.shape
+    out = torch.empty((L, hq * d), dtype=torch.bfloat16, device=q.device)
+    _lib.call("scmx_attn_prefill", _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache), _lib.ptr(out), L, int(off), hq, hk, d,
+              rows, float(scale if scale is not None else d ** -0.5), _lib.stream())
+    return out
+
+
 def attn_decode_qkv(y, qn, kn, eps, hq, hk, d, kcache, vcache, pos, inv_freq, scale=None):
     """qkv_headnorm_rope at L = 1 followed by attn_decode, in one launch and with the same bits: y bf16
     [1, (hq + 2 hk) d] -> bf16 [1, hq * d]; the token's k and v land in row pos of the caches.  pos: int, or an int64

@@ -20,16 +20,20 @@ def default_format_afterwards():
 
 @pytest.fixture(scope="module")
 def tiny():
+    return make_tiny(4, 2, 64)
+
+
+def make_tiny(hq, hk, head_dim):
     from mxfp4_int8_m5_amd import fused_qwen3 as Q, sc_weights as W
-    args = Q.Qwen3Args(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
-                       num_key_value_heads=2, head_dim=64, vocab_size=320, rope_theta=1e4)
+    args = Q.Qwen3Args(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=hq,
+                       num_key_value_heads=hk, head_dim=head_dim, vocab_size=320, rope_theta=1e4)
     g = torch.Generator().manual_seed(0)
     rnd = lambda *s, sc=1.0: torch.randn(*s, generator=g) * sc   # noqa: E731
     state = {"model.embed_tokens.weight": rnd(args.vocab_size, args.hidden_size),
              "model.norm.weight": 1 + rnd(args.hidden_size, sc=0.1)}
-    shapes = {"self_attn.q_proj": (256, 256), "self_attn.k_proj": (128, 256), "self_attn.v_proj": (128, 256),
-              "self_attn.o_proj": (256, 256), "mlp.gate_proj": (512, 256), "mlp.up_proj": (512, 256),
-              "mlp.down_proj": (256, 512)}
+    shapes = {"self_attn.q_proj": (hq * head_dim, 256), "self_attn.k_proj": (hk * head_dim, 256),
+              "self_attn.v_proj": (hk * head_dim, 256), "self_attn.o_proj": (256, hq * head_dim),
+              "mlp.gate_proj": (512, 256), "mlp.up_proj": (512, 256), "mlp.down_proj": (256, 512)}
     for i in range(args.num_hidden_layers):
         p = f"model.layers.{i}."
         for n in ("input_layernorm", "post_attention_layernorm"):
@@ -100,6 +104,26 @@ def test_prefill_against_float_model(tiny, epilogue):
     ref = float_model(Q, args, state, packed, ids)
     assert h.shape == ref.shape
     assert rel(h, ref) < 3e-2, rel(h, ref)       # two blocks of INT8 activations + bf16 residual stream
+
+
+def test_prefill_with_this_librarys_attention_kernel():
+    """Head dim 128: the prefill runs scmx_attn_prefill; against the float model, against the same driver on torch's
+    attention op, and a second chunk appended behind the first (attention at an offset) against one pass over both."""
+    Q, args, state, packed = make_tiny(4, 2, 128)
+    ids = torch.randint(0, args.vocab_size, (200,), generator=torch.Generator().manual_seed(21)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    assert m.attn_kernel
+    h = m.hidden(ids)
+    ref = float_model(Q, args, state, packed, ids.cpu())
+    assert rel(h, ref) < 4e-2, rel(h, ref)
+    m2 = Q.FusedQwen3(args, state, packed)
+    m2.attn_kernel = False
+    assert rel(h, m2.hidden(ids)) < 1e-2
+    cache = m.make_cache(256)
+    first = m.hidden(ids[:130], cache)
+    second = m.hidden(ids[130:], cache)
+    assert cache[0].offset == 200
+    assert torch.equal(first, h[:130]) and rel(second, h[130:]) < 1e-2
 
 
 def test_resident_int8_weights_give_the_same_result(tiny):
@@ -276,6 +300,36 @@ def test_fused_attention_decoder_equals_the_two_kernel_decoder(tiny, graphs):
         assert c1[0].offset == c2[0].offset == j + 1
         assert torch.equal(a, b), j
     assert all(torch.equal(x.k, z.k) and torch.equal(x.v, z.v) for x, z in zip(c1, c2))
+
+
+@pytest.mark.parametrize("hq,hk,L,off,rows", [(16, 8, 2048, 0, 2048), (4, 4, 300, 0, 512), (8, 2, 70, 33, 128),
+                                               (2, 1, 1, 0, 4), (6, 3, 129, 1000, 1200), (4, 2, 64, 64, 128)])
+def test_attn_prefill_against_torch(hq, hk, L, off, rows):
+    """Causal attention of L new tokens behind `off` cached ones (head dim 128): float32 softmax(q k^T) v of the same
+    bf16 inputs in torch within 1e-2 (bf16 probabilities and output); ragged last query and key tiles, grouped
+    heads, a cache longer than what is valid (rows past off + L hold NaN and must not be read into the result)."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    d = 128
+    g = torch.Generator(device="cuda").manual_seed(L + off)
+    q = torch.randn(L, hq, d, device="cuda", generator=g).to(torch.bfloat16)
+    kc = torch.randn(hk, rows, d, device="cuda", generator=g).to(torch.bfloat16)
+    vc = torch.randn(hk, rows, d, device="cuda", generator=g).to(torch.bfloat16)
+    kc[:, off + L:] = float("nan")
+    vc[:, off + L:] = float("nan")
+    n = off + L
+    rep = hq // hk
+    kf = kc[:, :n].float().repeat_interleave(rep, 0)
+    vf = vc[:, :n].float().repeat_interleave(rep, 0)
+    s = torch.einsum("lhd,hnd->hln", q.float(), kf) * d ** -0.5
+    mask = torch.arange(n, device="cuda")[None, :] <= (off + torch.arange(L, device="cuda"))[:, None]
+    p = torch.softmax(s.masked_fill(~mask[None], float("-inf")), -1)
+    ref = torch.einsum("hln,hnd->lhd", p, vf).reshape(L, hq * d)
+    o = S.attn_prefill(q.transpose(0, 1), kc, vc, off)          # the [hq, L, d] view, as the norm kernel hands it over
+    assert o.shape == (L, hq * d) and not torch.isnan(o).any()
+    assert rel(o, ref) < 1e-2, rel(o, ref)
+    assert torch.equal(S.attn_prefill(q.transpose(0, 1).contiguous(), kc, vc, off), o)     # head-major storage: copied
+    with pytest.raises(ValueError):
+        S.attn_prefill(q.transpose(0, 1), kc, vc, rows - L + 1)
 
 
 def test_packed_output_head(tiny):
