@@ -127,15 +127,16 @@ __global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __r
             const uint8_t* vs = smem[t & 1] + FA_KBYTES;
             f32x16 sacc[2];
 #pragma unroll
-            for (int blk = 0; blk < 2; ++blk) {
+            for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sacc[blk][r] = 0.0f;
 #pragma unroll
-                for (int s = 0; s < FA_D / 16; ++s) {
+            for (int s = 0; s < FA_D / 16; ++s)   // the two key blocks are independent accumulation chains: alternate them
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk) {
                     const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (blk * 32 + ln) * FA_KROW + 32 * s + 16 * h);
                     sacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[s], sacc[blk], 0, 0, 0);
                 }
-            }
             // running maximum of the raw scores; tiles that reach past the wave's first query are masked first
             if (kv0 + FA_BN - 1 > off + qw0) {
                 const int limit = off + qw0 + ln - kv0;   // keys with tile index <= limit are visible to this query
@@ -171,19 +172,20 @@ __global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __r
                     }
             l = l * alpha + ls;
             const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;   // no query's maximum moved: skip
+            if (rescale) {
 #pragma unroll
-            for (int db = 0; db < FA_D / 32; ++db) {
-                if (rescale) {
+                for (int db = 0; db < FA_D / 32; ++db)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
-                }
+            }
 #pragma unroll
-                for (int s = 0; s < FA_BN / 16; ++s) {
+            for (int s = 0; s < FA_BN / 16; ++s)   // four independent chains (head-dimension blocks) per key slice
+#pragma unroll
+                for (int db = 0; db < FA_D / 32; ++db) {
                     // keys 16s + 4h + (0..3) and 16s + 8 + 4h + (0..3) of head-dimension row db * 32 + ln
                     const bf16x8 a = *reinterpret_cast<const bf16x8*>(vs + (db * 32 + ln) * FA_VROW + 32 * s + 16 * h);
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[s], o[db], 0, 0, 0);
                 }
-            }
         }
         if (t + 1 < ntile) {
             store_tile(next, (t + 1) & 1);
