@@ -2,8 +2,11 @@
 // out[i] = softmax(q[i] . K[0 .. off+i]^T * scale) V[0 .. off+i] per query head, grouped-query sharing of the KV heads.
 //
 // The linear layers are the product here; this kernel exists because the attention between them is a third of the
-// prefill time with the array library's kernel.  One workgroup of four waves owns 128 consecutive queries of one head
-// (32 per wave) and walks the keys in tiles of 64 with a running maximum and sum (one pass over K and V).
+// prefill time with the array library's kernel.  One workgroup of four waves owns 64 consecutive queries of one head:
+// two blocks of 32 queries times two halves of the keys.  The keys are walked in pairs of 64-key tiles with a running
+// maximum and sum (one pass over K and V); wave (block, half) multiplies the pair's tile `half`, and the two halves
+// of a block are merged through LDS at the end.  Splitting the keys inside the workgroup halves the longest serial
+// chain (the last query tile sees every key) and puts two workgroups, i.e. two waves per SIMD, on a CU.
 //
 // Everything is computed transposed, so that no operand has to change lanes between the two matrix products:
 //   S^T = K Q^T    (v_mfma_f32_32x32x16_bf16: rows = keys, columns = queries, contraction over the head dimension)
@@ -16,8 +19,8 @@
 // head-dimension index, 144 bytes), written as pairs of keys so that a wave's LDS stores cover distinct words; inside
 // every 16-key slice the middle two groups of four keys change places, which puts the 8 keys of a lane half (4h + r
 // and 8 + 4h + r) next to each other: one 16-byte read per fragment.
-// Tiles are double-buffered in LDS and their global loads run two tiles ahead in two register sets, one barrier per
-// tile.  Query tiles are launched last to first (the last one sees the most keys).
+// A pair of tiles is single-buffered in LDS; the global loads of the next pair are in flight in registers while the
+// current one is multiplied (two barriers per pair, which the CU's other workgroup fills).  Query tiles are launched last to first (the last one sees the most keys).
 #include "scmx_common.h"
 
 namespace scmx {
@@ -26,14 +29,14 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int FA_NT = 256;                  // four waves
-constexpr int FA_BM = 128, FA_BN = 64, FA_D = 128;
+constexpr int FA_NT = 256;                  // four waves: (query block, key half)
+constexpr int FA_BM = 64, FA_BN = 64, FA_D = 128;
 constexpr int FA_KROW = FA_D * 2 + 16;      // bytes per K row in LDS
 constexpr int FA_VROW = FA_BN * 2 + 16;     // bytes per V^T row in LDS
 constexpr int FA_KBYTES = FA_BN * FA_KROW;
 constexpr int FA_VBYTES = FA_D * FA_VROW;
 
-__global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
+__global__ __launch_bounds__(FA_NT, 2) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
                                                              const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
                                                              int L, int off, int hq, int hk, int rows, float scale_log2) {
     __shared__ __attribute__((aligned(16))) uint8_t smem[2][FA_KBYTES + FA_VBYTES];
@@ -41,7 +44,8 @@ __global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __r
     const int num_qt = (L + FA_BM - 1) / FA_BM;
     const int qt = num_qt - 1 - int(blockIdx.x);
     const int head = blockIdx.y, kvh = head / (hq / hk);
-    const int q0 = qt * FA_BM, qw0 = q0 + wave * 32;
+    const int qb = wave & 1, kh = wave >> 1;   // query block and key half of this wave
+    const int q0 = qt * FA_BM, qw0 = q0 + qb * 32;
     const int n = off + L;   // valid cache rows
 
     // this lane's query as the column operand of S^T: 8 consecutive head-dimension values per 16-wide slice
@@ -63,46 +67,39 @@ __global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __r
     const uint16_t* kb = kc + size_t(kvh) * rows * FA_D;
     const uint16_t* vb = vc + size_t(kvh) * rows * FA_D;
 
-    // staging: K as 16-byte pieces (key = c / 16, piece = c % 16), V as pairs of keys (pair = c % 32, piece = c / 32)
-    constexpr int KJ = FA_BN * 16 / FA_NT, VJ = (FA_BN / 2) * 16 / FA_NT;
-    struct Staged {
-        u32x4 kr[KJ], va[VJ], vb2[VJ];
-    };
-    Staged r0, r1;   // tile k waits in set k % 2 from two iterations before it is multiplied
-    auto load_tile = [&](Staged& st, int t) {
-        u32x4(&kr)[KJ] = st.kr;
-        u32x4(&va)[VJ] = st.va;
-        u32x4(&vb2)[VJ] = st.vb2;
+    const int npair = (ntile + 1) / 2;
+
+    // staging of a pair of tiles: K as 16-byte pieces (tile = c / 1024, key = c / 16 % 64, piece = c % 16), V as pairs of
+    // keys (tile = c / 512, pair = c % 32, piece = c / 32 % 16)
+    constexpr int KJ = 2 * FA_BN * 16 / FA_NT, VJ = 2 * (FA_BN / 2) * 16 / FA_NT;
+    u32x4 kr[KJ], va[VJ], vb2[VJ];
+    auto load_pair = [&](int i) {
 #pragma unroll
         for (int j = 0; j < KJ; ++j) {
             const int c = tid + FA_NT * j;
-            const int key = min(t * FA_BN + c / 16, n - 1);
+            const int key = min((2 * i + c / 1024) * FA_BN + (c / 16) % FA_BN, n - 1);
             kr[j] = *reinterpret_cast<const u32x4*>(kb + size_t(key) * FA_D + (c % 16) * 8);
         }
 #pragma unroll
         for (int j = 0; j < VJ; ++j) {
             const int c = tid + FA_NT * j;
-            const int key = t * FA_BN + 2 * (c % 32);
-            const int piece = c / 32;
+            const int key = (2 * i + c / 512) * FA_BN + 2 * (c % 32);
+            const int piece = (c / 32) % 16;
             va[j] = *reinterpret_cast<const u32x4*>(vb + size_t(min(key, n - 1)) * FA_D + piece * 8);
             vb2[j] = *reinterpret_cast<const u32x4*>(vb + size_t(min(key + 1, n - 1)) * FA_D + piece * 8);
         }
     };
-    auto store_tile = [&](const Staged& st, int buf) {
-        const u32x4(&kr)[KJ] = st.kr;
-        const u32x4(&va)[VJ] = st.va;
-        const u32x4(&vb2)[VJ] = st.vb2;
-        uint8_t* ks = smem[buf];
-        uint8_t* vs = smem[buf] + FA_KBYTES;
+    auto store_pair = [&]() {
 #pragma unroll
         for (int j = 0; j < KJ; ++j) {
             const int c = tid + FA_NT * j;
-            *reinterpret_cast<u32x4*>(ks + (c / 16) * FA_KROW + (c % 16) * 16) = kr[j];
+            *reinterpret_cast<u32x4*>(smem[c / 1024] + ((c / 16) % FA_BN) * FA_KROW + (c % 16) * 16) = kr[j];
         }
 #pragma unroll
         for (int j = 0; j < VJ; ++j) {
             const int c = tid + FA_NT * j;
-            const int pair = c % 32, piece = c / 32;
+            uint8_t* vs = smem[c / 512] + FA_KBYTES;
+            const int pair = c % 32, piece = (c / 32) % 16;
             const int kk = 2 * pair;   // first key of the pair; its place in the row: bits 2 and 3 of the key index swapped
             const int place = (kk & ~12) | ((kk & 4) << 1) | ((kk & 8) >> 1);
 #pragma unroll
@@ -113,18 +110,16 @@ __global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __r
         }
     };
 
-    load_tile(r0, 0);
-    if (ntile > 1) load_tile(r1, 1);
-    store_tile(r0, 0);
-    if (ntile > 2) load_tile(r0, 2);
+    load_pair(0);
+    store_pair();
     __syncthreads();
-    // one iteration: multiply tile t out of its LDS buffer, then move tile t + 1 from its register set into the other
-    // buffer (last read one barrier ago) and reuse the set for the loads of tile t + 3
-    auto iteration = [&](int t, Staged& next) {
+    if (npair > 1) load_pair(1);
+    for (int i = 0; i < npair; ++i) {
+        const int t = 2 * i + kh;
         const int kv0 = t * FA_BN;
         if (kv0 <= off + qw0 + 31) {   // some key of the tile is visible to some query of this wave
-            const uint8_t* ks = smem[t & 1];
-            const uint8_t* vs = smem[t & 1] + FA_KBYTES;
+            const uint8_t* ks = smem[kh];
+            const uint8_t* vs = smem[kh] + FA_KBYTES;
             f32x16 sacc[2];
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk)
@@ -187,17 +182,36 @@ __global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __r
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[s], o[db], 0, 0, 0);
                 }
         }
-        if (t + 1 < ntile) {
-            store_tile(next, (t + 1) & 1);
-            if (t + 3 < ntile) load_tile(next, t + 3);
+        __syncthreads();   // every wave is done with the pair
+        if (i + 1 < npair) {
+            store_pair();
+            if (i + 2 < npair) load_pair(i + 2);   // the registers are free again: next loads go out before the barrier
+            __syncthreads();
         }
-        __syncthreads();
-    };
-    for (int t = 0; t < ntile; t += 2) {
-        iteration(t, r1);
-        if (t + 1 < ntile) iteration(t + 1, r0);
     }
 
+    // merge the two key halves of every query block: the second half parks its state in LDS, the first one folds it in
+    float* park = reinterpret_cast<float*>(&smem[0][0]) + qb * (FA_D / 32 * 16 + 2) * 64;
+    if (kh == 1) {
+#pragma unroll
+        for (int db = 0; db < FA_D / 32; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) park[(db * 16 + r) * 64 + lane] = o[db][r];
+        park[(FA_D / 32 * 16) * 64 + lane] = m;
+        park[(FA_D / 32 * 16 + 1) * 64 + lane] = l;
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    {
+        const float m2 = park[(FA_D / 32 * 16) * 64 + lane], l2 = park[(FA_D / 32 * 16 + 1) * 64 + lane];
+        const float mn = fmaxf(m, m2);
+        const float a1 = __builtin_amdgcn_exp2f((m - mn) * scale_log2), a2 = __builtin_amdgcn_exp2f((m2 - mn) * scale_log2);
+        l = l * a1 + l2 * a2;
+#pragma unroll
+        for (int db = 0; db < FA_D / 32; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[db][r] = o[db][r] * a1 + park[(db * 16 + r) * 64 + lane] * a2;
+    }
     l += __shfl_xor(l, 32, WAVE);
     const float inv = 1.0f / l;
     const int query = qw0 + ln;
