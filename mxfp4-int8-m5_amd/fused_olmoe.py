@@ -111,6 +111,8 @@ class FusedOlmoe:
         k, v = c.update_and_fetch(k, v)
         if L == 1:
             return S.attn_decode(q, c.k, c.v, off + 1)
+        if q.shape[-1] == 128:   # this library's causal attention (head dim 128 only; q is copied to token-major)
+            return S.attn_prefill(q, c.k, c.v, off)
         if off == 0:
             o = TF.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)
         else:

@@ -410,9 +410,13 @@ def test_load_fused_in_a_family_format(tiny, tmp_path):
 
 @pytest.fixture(scope="module")
 def tiny_moe():
+    return make_tiny_moe(4)
+
+
+def make_tiny_moe(heads):
     from mxfp4_int8_m5_amd import fused_olmoe as O, sc_weights as W
-    args = O.OlmoeArgs(hidden_size=256, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4, num_experts=8,
-                       num_experts_per_tok=2, vocab_size=300)
+    args = O.OlmoeArgs(hidden_size=256, intermediate_size=128, num_hidden_layers=2, num_attention_heads=heads,
+                       num_experts=8, num_experts_per_tok=2, vocab_size=300)
     g = torch.Generator().manual_seed(10)
     rnd = lambda *s, sc=1.0: torch.randn(*s, generator=g) * sc   # noqa: E731
     D, Fi, E = args.hidden_size, args.intermediate_size, args.num_experts
@@ -488,6 +492,16 @@ def test_olmoe_prefill_against_float_model(tiny_moe, kw):
     h = m.hidden(ids.cuda())
     ref = moe_float_model(args, state, packed, ids, m.record)
     assert rel(h, ref) < 4e-2, rel(h, ref)
+
+
+def test_olmoe_prefill_with_head_dim_128():
+    """Two heads of 128: the prefill attention runs through scmx_attn_prefill (q copied to token-major first)."""
+    O, args, state, packed = make_tiny_moe(2)
+    ids = torch.randint(0, args.vocab_size, (70,), generator=torch.Generator().manual_seed(13))
+    m = O.FusedOlmoe(args, state, packed, tile=64)
+    m.record = []
+    h = m.hidden(ids.cuda())
+    assert rel(h, moe_float_model(args, state, packed, ids, m.record)) < 4e-2
 
 
 @pytest.mark.parametrize("fuse", [False, "o", True])
