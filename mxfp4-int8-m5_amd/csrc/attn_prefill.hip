@@ -2,11 +2,11 @@
 // out[i] = softmax(q[i] . K[0 .. off+i]^T * scale) V[0 .. off+i] per query head, grouped-query sharing of the KV heads.
 //
 // The linear layers are the product here; this kernel exists because the attention between them is a third of the
-// prefill time with the array library's kernel.  One workgroup of four waves owns 64 consecutive queries of one head:
-// two blocks of 32 queries times two halves of the keys.  The keys are walked in pairs of 64-key tiles with a running
+// prefill time with the array library's kernel.  One workgroup of eight waves owns 128 consecutive queries of one head:
+// four blocks of 32 queries times two halves of the keys.  The keys are walked in pairs of 64-key tiles with a running
 // maximum and sum (one pass over K and V); wave (block, half) multiplies the pair's tile `half`, and the two halves
 // of a block are merged through LDS at the end.  Splitting the keys inside the workgroup halves the longest serial
-// chain (the last query tile sees every key) and puts two workgroups, i.e. two waves per SIMD, on a CU.
+// chain (the last query tile sees every key) and puts two waves on every SIMD, and eight waves share what is staged.
 //
 // Everything is computed transposed, so that no operand has to change lanes between the two matrix products:
 //   S^T = K Q^T    (v_mfma_f32_32x32x16_bf16: rows = keys, columns = queries, contraction over the head dimension)
@@ -19,8 +19,8 @@
 // head-dimension index, 144 bytes), written as pairs of keys so that a wave's LDS stores cover distinct words; inside
 // every 16-key slice the middle two groups of four keys change places, which puts the 8 keys of a lane half (4h + r
 // and 8 + 4h + r) next to each other: one 16-byte read per fragment.
-// A pair of tiles is single-buffered in LDS; the global loads of the next pair are in flight in registers while the
-// current one is multiplied (two barriers per pair, which the CU's other workgroup fills).  Query tiles are launched last to first (the last one sees the most keys).
+// Pairs of tiles are double-buffered in LDS and the global loads of the pair after the next one are in flight in
+// registers while the current one is multiplied: one barrier per pair.  Query tiles are launched last to first (the last one sees the most keys).
 #include "scmx_common.h"
 
 namespace scmx {
@@ -29,22 +29,22 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int FA_NT = 256;                  // four waves: (query block, key half)
-constexpr int FA_BM = 64, FA_BN = 64, FA_D = 128;
+constexpr int FA_NT = 512;                  // eight waves: (query block, key half)
+constexpr int FA_BM = 128, FA_BN = 64, FA_D = 128;
 constexpr int FA_KROW = FA_D * 2 + 16;      // bytes per K row in LDS
 constexpr int FA_VROW = FA_BN * 2 + 16;     // bytes per V^T row in LDS
 constexpr int FA_KBYTES = FA_BN * FA_KROW;
 constexpr int FA_VBYTES = FA_D * FA_VROW;
 
-__global__ __launch_bounds__(FA_NT, 2) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
+__global__ __launch_bounds__(FA_NT) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
                                                              const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
                                                              int L, int off, int hq, int hk, int rows, float scale_log2) {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[2][FA_KBYTES + FA_VBYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t smem[2][2][FA_KBYTES + FA_VBYTES];   // [buffer][tile of the pair]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, h = lane >> 5;
     const int num_qt = (L + FA_BM - 1) / FA_BM;
     const int qt = num_qt - 1 - int(blockIdx.x);
     const int head = blockIdx.y, kvh = head / (hq / hk);
-    const int qb = wave & 1, kh = wave >> 1;   // query block and key half of this wave
+    const int qb = wave & 3, kh = wave >> 2;   // query block and key half of this wave
     const int q0 = qt * FA_BM, qw0 = q0 + qb * 32;
     const int n = off + L;   // valid cache rows
 
@@ -89,16 +89,16 @@ __global__ __launch_bounds__(FA_NT, 2) void attn_prefill_kernel(const uint16_t* 
             vb2[j] = *reinterpret_cast<const u32x4*>(vb + size_t(min(key + 1, n - 1)) * FA_D + piece * 8);
         }
     };
-    auto store_pair = [&]() {
+    auto store_pair = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < KJ; ++j) {
             const int c = tid + FA_NT * j;
-            *reinterpret_cast<u32x4*>(smem[c / 1024] + ((c / 16) % FA_BN) * FA_KROW + (c % 16) * 16) = kr[j];
+            *reinterpret_cast<u32x4*>(smem[buf][c / 1024] + ((c / 16) % FA_BN) * FA_KROW + (c % 16) * 16) = kr[j];
         }
 #pragma unroll
         for (int j = 0; j < VJ; ++j) {
             const int c = tid + FA_NT * j;
-            uint8_t* vs = smem[c / 512] + FA_KBYTES;
+            uint8_t* vs = smem[buf][c / 512] + FA_KBYTES;
             const int pair = c % 32, piece = (c / 32) % 16;
             const int kk = 2 * pair;   // first key of the pair; its place in the row: bits 2 and 3 of the key index swapped
             const int place = (kk & ~12) | ((kk & 4) << 1) | ((kk & 8) >> 1);
@@ -111,15 +111,15 @@ __global__ __launch_bounds__(FA_NT, 2) void attn_prefill_kernel(const uint16_t* 
     };
 
     load_pair(0);
-    store_pair();
-    __syncthreads();
+    store_pair(0);
     if (npair > 1) load_pair(1);
+    __syncthreads();
     for (int i = 0; i < npair; ++i) {
         const int t = 2 * i + kh;
         const int kv0 = t * FA_BN;
         if (kv0 <= off + qw0 + 31) {   // some key of the tile is visible to some query of this wave
-            const uint8_t* ks = smem[kh];
-            const uint8_t* vs = smem[kh] + FA_KBYTES;
+            const uint8_t* ks = smem[i & 1][kh];
+            const uint8_t* vs = smem[i & 1][kh] + FA_KBYTES;
             f32x16 sacc[2];
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk)
@@ -182,16 +182,15 @@ __global__ __launch_bounds__(FA_NT, 2) void attn_prefill_kernel(const uint16_t* 
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[s], o[db], 0, 0, 0);
                 }
         }
-        __syncthreads();   // every wave is done with the pair
-        if (i + 1 < npair) {
-            store_pair();
-            if (i + 2 < npair) load_pair(i + 2);   // the registers are free again: next loads go out before the barrier
-            __syncthreads();
+        if (i + 1 < npair) {   // the other buffer was last read one barrier ago
+            store_pair((i + 1) & 1);
+            if (i + 2 < npair) load_pair(i + 2);   // the registers are free again
         }
+        __syncthreads();
     }
 
     // merge the two key halves of every query block: the second half parks its state in LDS, the first one folds it in
-    float* park = reinterpret_cast<float*>(&smem[0][0]) + qb * (FA_D / 32 * 16 + 2) * 64;
+    float* park = reinterpret_cast<float*>(&smem[0][0][0]) + qb * (FA_D / 32 * 16 + 2) * 64;
     if (kh == 1) {
 #pragma unroll
         for (int db = 0; db < FA_D / 32; ++db)
