@@ -2,7 +2,8 @@
  *
  * Every entry point enqueues HIP kernels on the caller's stream and returns at once (stream-ordered, no implicit
  * synchronisation).  Pointers are DEVICE pointers unless stated otherwise; the library never allocates or frees
- * device memory and keeps no state between calls, so it is reentrant.  Return value: 0 on success, a negative
+ * device memory and keeps no state between calls (beyond the per-device address of its constant SiLU lookup table,
+ * looked up once), so it is reentrant.  Return value: 0 on success, a negative
  * SCMX_ERR_* code otherwise, with a message available from scmx_last_error() (thread-local).
  *
  * Each declaration names the function of the reference (shinyoungkang1/mxfp4-int8-m5) it replaces, as file:line.
