@@ -43,14 +43,32 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
     const uint16_t* kbase = kc + size_t(kvh) * rows * D + 8 * c;
     const uint16_t* vbase = vc + size_t(kvh) * rows * D + 8 * c;
 
+    // Every lane of the workgroup runs the same number of trips (rows beyond n are skipped by predication), so the
+    // cross-lane sums below always see whole groups.
+    const int trips = (n + GROUPS - 1) / GROUPS;
+    constexpr int UN = 4;   // rows in flight per lane group: the K and V rows of UN steps are requested together
+    u32x4 kw[UN], vw[UN];
+    auto load_trip = [&](int t0) {
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int j = (t0 + u) * GROUPS + grp;
+            const size_t ro = size_t(j < n ? j : 0) * D;
+            kw[u] = *reinterpret_cast<const u32x4*>(kbase + ro);
+            vw[u] = *reinterpret_cast<const u32x4*>(vbase + ro);
+        }
+    };
+    load_trip(0);   // on their way while the fused variant prepares q and the new row
+
     if (FUSED) {
         constexpr int PER = D / 64;
         const int lane = tid & 63, wave = tid >> 6;
         const int newrow = n - 1;   // the position of the token being decoded
-        for (int i = tid; i < D / 2; i += ANT) sincosf(float(int64_t(newrow)) * x.inv_freq[i], &s_sin[i], &s_cos[i]);
-        __syncthreads();
-        if (wave < 3) {   // wave 0: q head, wave 1: k head, wave 2: v head
-            const int g = wave == 0 ? head : (wave == 1 ? hq + kvh : hq + hk + kvh);
+        // wave 3 computes the row's sines and cosines while waves 0 / 1 / 2 fetch and normalise the q / k / v head
+        float nv[PER];
+        const int g = wave == 0 ? head : (wave == 1 ? hq + kvh : hq + hk + kvh);
+        if (wave == 3) {
+            for (int i = lane; i < D / 2; i += 64) sincosf(float(int64_t(newrow)) * x.inv_freq[i], &s_sin[i], &s_cos[i]);
+        } else {
             float yv[PER];
             float ss = 0.0f;
 #pragma unroll
@@ -58,18 +76,22 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
                 yv[i] = bf16_to_f32(x.y[size_t(g) * D + PER * lane + i]);
                 ss = __fadd_rn(ss, __fmul_rn(yv[i], yv[i]));
             }
+            if (wave < 2) {
+                head_norm(yv, ss, PER, lane, D, wave == 0 ? x.qn : x.kn, x.eps, nv);
+            } else {
+#pragma unroll
+                for (int i = 0; i < PER; ++i) nv[i] = yv[i];
+            }
+        }
+        __syncthreads();
+        if (wave < 3) {
             const bool append = wave > 0 && head % (hq / hk) == 0;
             uint16_t* dst = (wave == 1 ? kc : vc) + (size_t(kvh) * rows + newrow) * D + PER * lane;
             auto emit = [&](int i, uint16_t b) {
                 s_new[wave][PER * lane + i] = b;
                 if (append) dst[i] = b;
             };
-            if (wave < 2) {
-                head_norm_rope(yv, ss, PER, lane, D, wave == 0 ? x.qn : x.kn, x.eps, s_sin, s_cos, emit);
-            } else {
-#pragma unroll
-                for (int i = 0; i < PER; ++i) emit(i, f32_to_bf16(yv[i]));
-            }
+            head_rope(nv, PER, lane, D, wave < 2 ? s_sin : nullptr, s_cos, emit);   // v passes through unrotated
         }
         __syncthreads();
     }
@@ -86,23 +108,15 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
     }
     float m = -3.0e38f, l = 0.0f;
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    // Every lane of the workgroup runs the same number of trips (rows beyond n are skipped by predication), so the
-    // cross-lane sums below always see whole groups.
-    const int trips = (n + GROUPS - 1) / GROUPS;
-    constexpr int UN = 4;   // rows in flight per lane group: the K and V rows of UN steps are requested together
     for (int t0 = 0; t0 < trips; t0 += UN) {
-        u32x4 kw[UN], vw[UN];
+        if (t0 > 0) load_trip(t0);
+        if (FUSED) {   // the new row comes from LDS, not from the cache being appended to
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int j = (t0 + u) * GROUPS + grp;
-            if (FUSED && j == n - 1) {   // the new row comes from LDS, not from the cache being appended to
-                kw[u] = *reinterpret_cast<const u32x4*>(&s_new[1][8 * c]);
-                vw[u] = *reinterpret_cast<const u32x4*>(&s_new[2][8 * c]);
-            } else {
-                const size_t ro = size_t(j < n ? j : 0) * D;
-                kw[u] = *reinterpret_cast<const u32x4*>(kbase + ro);
-                vw[u] = *reinterpret_cast<const u32x4*>(vbase + ro);
-            }
+            for (int u = 0; u < UN; ++u)
+                if ((t0 + u) * GROUPS + grp == n - 1) {
+                    kw[u] = *reinterpret_cast<const u32x4*>(&s_new[1][8 * c]);
+                    vw[u] = *reinterpret_cast<const u32x4*>(&s_new[2][8 * c]);
+                }
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {

@@ -212,27 +212,40 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
     return v;
 }
 
-// Per-head RMSNorm of one q or k head held by one wave, then (sn != nullptr) the rotary embedding: the lane holds the
-// bf16-valued elements per*lane .. per*lane + per - 1 of the head in yv and their sum of squares in ss; sn / cs are
-// the d / 2 sines and cosines of the row's position.  emit(i, value) receives the bf16 result of element per*lane + i.
-// Shared by the row kernel and the fused decode attention so that both give the same bits.
+// Per-head RMSNorm of one q or k head held by one wave: the lane holds the bf16-valued elements per*lane ..
+// per*lane + per - 1 of the head in yv and their sum of squares in ss; nv receives the normalised values (bf16-valued).
+__device__ __forceinline__ void head_norm(const float* yv, float ss, int per, int lane, int d,
+                                          const uint16_t* __restrict__ w, float eps, float* nv) {
+    ss = wave_sum(ss);
+    const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
+    for (int i = 0; i < per; ++i)
+        nv[i] = round_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
+}
+// The rotary embedding of such a head (sn / cs: the d / 2 sines and cosines of the row's position; sn == nullptr: no
+// rotation).  emit(i, value) receives the bf16 result of element per*lane + i.
+template <typename Emit>
+__device__ __forceinline__ void head_rope(const float* nv, int per, int lane, int d, const float* sn, const float* cs,
+                                          Emit&& emit) {
+    for (int i = 0; i < per; ++i) {
+        float v = nv[i];
+        if (sn) {
+            // element e = per*lane + i pairs with e +- d/2, held by lane +- 32 at the same i
+            const float other = __shfl_xor(v, 32, WAVE);
+            const int e = (per * lane + i) % (d / 2);
+            v = lane < 32 ? __fsub_rn(__fmul_rn(v, cs[e]), __fmul_rn(other, sn[e]))
+                          : __fadd_rn(__fmul_rn(v, cs[e]), __fmul_rn(other, sn[e]));
+        }
+        emit(i, f32_to_bf16(v));
+    }
+}
+// Both in sequence.  Shared by the row kernel and the fused decode attention so that both give the same bits.
 template <typename Emit>
 __device__ __forceinline__ void head_norm_rope(const float* yv, float ss, int per, int lane, int d,
                                                const uint16_t* __restrict__ w, float eps, const float* sn,
                                                const float* cs, Emit&& emit) {
-    ss = wave_sum(ss);
-    const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
-    for (int i = 0; i < per; ++i) {
-        float nv = round_bf16(__fmul_rn(bf16_to_f32(w[per * lane + i]), round_bf16(__fmul_rn(yv[i], inv))));
-        if (sn) {
-            // element e = per*lane + i pairs with e +- d/2, held by lane +- 32 at the same i
-            const float other = __shfl_xor(nv, 32, WAVE);
-            const int e = (per * lane + i) % (d / 2);
-            nv = lane < 32 ? __fsub_rn(__fmul_rn(nv, cs[e]), __fmul_rn(other, sn[e]))
-                           : __fadd_rn(__fmul_rn(nv, cs[e]), __fmul_rn(other, sn[e]));
-        }
-        emit(i, f32_to_bf16(nv));
-    }
+    float nv[8];
+    head_norm(yv, ss, per, lane, d, w, eps, nv);
+    head_rope(nv, per, lane, d, sn, cs, emit);
 }
 
 // Symmetric INT8 code of v at inverse scale qi: clamp(rint(v * qi), +-127).
