@@ -129,18 +129,23 @@ int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float*
  * [hq, d], caches bf16 [hk, cache_rows, d] of which the first n rows are valid; n = *pos_dev + 1 when pos_dev != NULL
  * (device-resident position, for graph replay).  d in {64, 128, 256}.  Takes the place of the
  * array library's scaled-dot-product attention at L = 1 in the decode step (e2e/decode.py:1-5, e2e/fused_qwen3.py:
- * 216-222), so that the step is a fixed launch sequence. */
+ * 216-222), so that the step is a fixed launch sequence.  splits > 1 (at most 64; for long contexts): the valid rows
+ * are cut into `splits` ranges, one workgroup per head and range, and a second launch merges the ranges' results out of
+ * `workspace`, float [splits * hq * (d + 2)]; splits == 1 needs no workspace (NULL). */
 int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, const int64_t* pos_dev, int n,
-                     uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, void* stream);
+                     uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, float* workspace, int splits,
+                     void* stream);
 
 /* scmx_qkv_headnorm_rope at L = 1 and scmx_attn_decode in one launch: y bf16 [(hq + 2 hk) * d] is the token's q|k|v
  * row from the qkv projection; per-head RMSNorm of q and k, rotary embedding at position p (*pos_dev, or pos0 when
- * pos_dev is NULL), append of k and v to row p of the caches, attention over rows 0..p.  Same bits as the two calls.
+ * pos_dev is NULL), append of k and v to row p of the caches, attention over rows 0..p.  Same bits as the two calls
+ * (with the same `splits`; workspace / splits as for scmx_attn_decode).
  * One launch less per block of the batch-1 decode step (e2e/decode.py:51-82; the array ops it stands for are
  * e2e/fused_qwen3.py:216-222). */
 int scmx_attn_decode_qkv(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps, const float* inv_freq,
                          const int64_t* pos_dev, int64_t pos0, uint16_t* kcache, uint16_t* vcache, uint16_t* out,
-                         int hq, int hk, int d, int cache_rows, float scale, void* stream);
+                         int hq, int hk, int d, int cache_rows, float scale, float* workspace, int splits,
+                         void* stream);
 
 /* Causal attention of L new tokens against a KV cache that holds `off` earlier rows followed by the L new ones:
  * q bf16 [L, hq, d] (token-major, as scmx_qkv_headnorm_rope writes it with q_token_major), caches bf16

@@ -33,9 +33,9 @@ SIGNATURES = {
     "scmx_res_norm_quant": (_I, [_P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _P]),
     "scmx_swiglu_quant": (_I, [_P, _P, _P, _P, _P, _I, _I, _P]),
     "scmx_qkv_headnorm": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P]),
-    "scmx_attn_decode": (_I, [_P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P]),
+    "scmx_attn_decode": (_I, [_P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P, _I, _P]),
     "scmx_attn_prefill": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P]),
-    "scmx_attn_decode_qkv": (_I, [_P, _P, _P, _F, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _F, _P]),
+    "scmx_attn_decode_qkv": (_I, [_P, _P, _P, _F, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _F, _P, _I, _P]),
     "scmx_qkv_headnorm_rope": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _L, _I, _I, _P]),
     "scmx_qkv_fullnorm": (_I, [_P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P]),
     "scmx_gemv": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _F, _I, _I, _I, _P, _I, _I, _I, _P]),

@@ -5,12 +5,15 @@
 // captured launch serves every position.  One workgroup per query head.  A row of K or V (d bf16 values) is read by
 // d / 8 lanes, 16 bytes each; such a lane group walks every (groups)-th row with a running maximum, sum and
 // weighted value chunk (one pass over K and V, both rows of a step in flight together), and the groups' partial
-// results are merged through LDS.  Accumulation is float32, the output bf16.
+// results are merged through LDS.  Accumulation is float32, the output bf16.  For long contexts the rows of a head
+// are cut into several ranges, one workgroup each (16 workgroups alone read a long cache at a fraction of the memory
+// bandwidth), and a small second kernel merges the ranges' results.
 #include "scmx_common.h"
 
 namespace scmx {
 
 constexpr int ANT = 256;
+constexpr int ATTN_SINGLE_MAX = 512;   // rows up to which a split launch falls back to one workgroup per head
 
 // What the fused variant needs besides the attention operands: the token's q|k|v row as the qkv projection wrote it,
 // the per-head norm weights and the rotary frequencies.
@@ -31,7 +34,7 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
                                                          uint16_t* __restrict__ vc,
                                                          const int64_t* __restrict__ pos_dev, int n0,
                                                          uint16_t* __restrict__ out, int hq, int hk, int rows, float scale,
-                                                         const QkvArgs x) {
+                                                         const QkvArgs x, float* __restrict__ partial) {
     constexpr int LPR = D / 8;              // lanes per cache row
     constexpr int GROUPS = ANT / LPR;       // lane groups per workgroup, each walking its own rows
     __shared__ float s_m[GROUPS], s_l[GROUPS], s_acc[GROUPS][D];
@@ -43,16 +46,25 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
     const uint16_t* kbase = kc + size_t(kvh) * rows * D + 8 * c;
     const uint16_t* vbase = vc + size_t(kvh) * rows * D + 8 * c;
 
-    // Every lane of the workgroup runs the same number of trips (rows beyond n are skipped by predication), so the
+    // gridDim.y > 1: the valid rows are cut into gridDim.y equal ranges, one per workgroup of a head; every workgroup
+    // leaves its unnormalised result, maximum and sum in `partial` and a second kernel merges them.
+    // A context of at most ATTN_SINGLE_MAX rows is read fastest by one workgroup per head: range 0 then takes all of
+    // it and writes the output, the other workgroups leave at once and the merge kernel finds nothing to do.
+    const bool single = gridDim.y == 1 || n <= ATTN_SINGLE_MAX;
+    if (single && blockIdx.y > 0) return;
+    const int nsplit = single ? 1 : int(gridDim.y);
+    const int chunk = (n + nsplit - 1) / nsplit;
+    const int row0 = int(blockIdx.y) * chunk, row1 = min(n, row0 + chunk);   // this workgroup's rows [row0, row1)
+    // Every lane of the workgroup runs the same number of trips (rows beyond row1 are skipped by predication), so the
     // cross-lane sums below always see whole groups.
-    const int trips = (n + GROUPS - 1) / GROUPS;
+    const int trips = (max(row1 - row0, 0) + GROUPS - 1) / GROUPS;
     constexpr int UN = 4;   // rows in flight per lane group: the K and V rows of UN steps are requested together
     u32x4 kw[UN], vw[UN];
     auto load_trip = [&](int t0) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int j = (t0 + u) * GROUPS + grp;
-            const size_t ro = size_t(j < n ? j : 0) * D;
+            const int j = row0 + (t0 + u) * GROUPS + grp;
+            const size_t ro = size_t(j < row1 ? j : 0) * D;
             kw[u] = *reinterpret_cast<const u32x4*>(kbase + ro);
             vw[u] = *reinterpret_cast<const u32x4*>(vbase + ro);
         }
@@ -85,7 +97,7 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
         }
         __syncthreads();
         if (wave < 3) {
-            const bool append = wave > 0 && head % (hq / hk) == 0;
+            const bool append = wave > 0 && head % (hq / hk) == 0 && blockIdx.y == 0;
             uint16_t* dst = (wave == 1 ? kc : vc) + (size_t(kvh) * rows + newrow) * D + PER * lane;
             auto emit = [&](int i, uint16_t b) {
                 s_new[wave][PER * lane + i] = b;
@@ -113,14 +125,14 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
         if (FUSED) {   // the new row comes from LDS, not from the cache being appended to
 #pragma unroll
             for (int u = 0; u < UN; ++u)
-                if ((t0 + u) * GROUPS + grp == n - 1) {
+                if (row0 + (t0 + u) * GROUPS + grp == n - 1) {
                     kw[u] = *reinterpret_cast<const u32x4*>(&s_new[1][8 * c]);
                     vw[u] = *reinterpret_cast<const u32x4*>(&s_new[2][8 * c]);
                 }
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const bool ok = (t0 + u) * GROUPS + grp < n;
+            const bool ok = row0 + (t0 + u) * GROUPS + grp < row1;
             float s = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -159,20 +171,60 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
             num += w * s_acc[g][e];
             den += w * s_l[g];
         }
-        out[size_t(head) * D + e] = f32_to_bf16(num / den);
+        if (single) {
+            out[size_t(head) * D + e] = f32_to_bf16(num / den);
+        } else {   // num and den are relative to mx; a range without rows leaves mx = -3e38, den = 0
+            float* pw = partial + (size_t(head) * gridDim.y + blockIdx.y) * (D + 2);
+            pw[e] = num;
+            if (e == 0) {
+                pw[D] = mx;
+                pw[D + 1] = den;
+            }
+        }
     }
+}
+
+// Merge of the per-range results of one head: out = sum_s w_s num_s / sum_s w_s den_s with w_s = exp(m_s - max m).
+template <int D>
+__global__ __launch_bounds__(D) void attn_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out,
+                                                     int splits, const int64_t* __restrict__ pos_dev, int n0, int rows) {
+    if (min(rows, pos_dev ? int(pos_dev[0]) + 1 : n0) <= ATTN_SINGLE_MAX) return;   // range 0 wrote the output itself
+    const int head = blockIdx.x, e = threadIdx.x;
+    const float* pw = partial + size_t(head) * splits * (D + 2);
+    float mx = -3.0e38f;
+    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, pw[s * (D + 2) + D]);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < splits; ++s) {
+        const float w = __expf(pw[s * (D + 2) + D] - mx);
+        num += w * pw[s * (D + 2) + e];
+        den += w * pw[s * (D + 2) + D + 1];
+    }
+    out[size_t(head) * D + e] = f32_to_bf16(num / den);
 }
 
 template <bool FUSED>
 static void launch_attn(int d, hipStream_t st, const uint16_t* q, uint16_t* kc, uint16_t* vc, const int64_t* pos_dev, int n,
-                        uint16_t* out, int hq, int hk, int rows, float scale, const QkvArgs& x) {
-    const dim3 grid(hq), wg(ANT);
-    if (d == 64)
-        attn_decode_kernel<64, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x);
-    else if (d == 128)
-        attn_decode_kernel<128, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x);
-    else
-        attn_decode_kernel<256, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x);
+                        uint16_t* out, int hq, int hk, int rows, float scale, const QkvArgs& x, float* partial, int splits) {
+    const dim3 grid(hq, splits), wg(ANT);
+    if (d == 64) {
+        attn_decode_kernel<64, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x, partial);
+        if (splits > 1) attn_merge_kernel<64><<<dim3(hq), dim3(64), 0, st>>>(partial, out, splits, pos_dev, n, rows);
+    } else if (d == 128) {
+        attn_decode_kernel<128, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x, partial);
+        if (splits > 1) attn_merge_kernel<128><<<dim3(hq), dim3(128), 0, st>>>(partial, out, splits, pos_dev, n, rows);
+    } else {
+        attn_decode_kernel<256, FUSED><<<grid, wg, 0, st>>>(q, kc, vc, pos_dev, n, out, hq, hk, rows, scale, x, partial);
+        if (splits > 1) attn_merge_kernel<256><<<dim3(hq), dim3(256), 0, st>>>(partial, out, splits, pos_dev, n, rows);
+    }
+}
+
+// The row ranges of a split launch: `workspace` holds splits * hq * (d + 2) floats.
+static int check_split(const char* who, const float* workspace, int splits) {
+    if (splits < 1 || splits > 64 || (splits > 1 && (!workspace || uintptr_t(workspace) % 4))) {
+        set_error("%s: splits must be 1..64 and need a float workspace of splits * hq * (d + 2) entries", who);
+        return SCMX_ERR_ARG;
+    }
+    return SCMX_OK;
 }
 
 }  // namespace scmx
@@ -192,7 +244,8 @@ static int check_attn(const char* who, int hq, int hk, int d, int cache_rows) {
 }
 
 extern "C" int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, const int64_t* pos_dev,
-                                int n, uint16_t* out, int hq, int hk, int d, int cache_rows, float scale, void* stream) {
+                                int n, uint16_t* out, int hq, int hk, int d, int cache_rows, float scale,
+                                float* workspace, int splits, void* stream) {
     if (!q || !kcache || !vcache || !out) {
         set_error("attn_decode: null pointer argument");
         return SCMX_ERR_ARG;
@@ -202,15 +255,16 @@ extern "C" int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const
         set_error("attn_decode: %d valid rows outside 1..%d", n, cache_rows);
         return SCMX_ERR_ARG;
     }
+    if (int rc = check_split("attn_decode", workspace, splits)) return rc;
     launch_attn<false>(d, (hipStream_t)stream, q, const_cast<uint16_t*>(kcache), const_cast<uint16_t*>(vcache), pos_dev, n,
-                       out, hq, hk, cache_rows, scale, QkvArgs{});
+                       out, hq, hk, cache_rows, scale, QkvArgs{}, workspace, splits);
     return check_launch("attn_decode");
 }
 
 extern "C" int scmx_attn_decode_qkv(const uint16_t* y, const uint16_t* qn, const uint16_t* kn, float eps,
                                     const float* inv_freq, const int64_t* pos_dev, int64_t pos0, uint16_t* kcache,
                                     uint16_t* vcache, uint16_t* out, int hq, int hk, int d, int cache_rows, float scale,
-                                    void* stream) {
+                                    float* workspace, int splits, void* stream) {
     if (!y || !qn || !kn || !inv_freq || !kcache || !vcache || !out) {
         set_error("attn_decode_qkv: null pointer argument");
         return SCMX_ERR_ARG;
@@ -224,7 +278,8 @@ extern "C" int scmx_attn_decode_qkv(const uint16_t* y, const uint16_t* qn, const
         set_error("attn_decode_qkv: position %lld outside a cache of %d rows", (long long)pos0, cache_rows);
         return SCMX_ERR_ARG;
     }
+    if (int rc = check_split("attn_decode_qkv", workspace, splits)) return rc;
     launch_attn<true>(d, (hipStream_t)stream, nullptr, kcache, vcache, pos_dev, int(pos0) + 1, out, hq, hk, cache_rows, scale,
-                      QkvArgs{y, qn, kn, inv_freq, eps});
+                      QkvArgs{y, qn, kn, inv_freq, eps}, workspace, splits);
     return check_launch("attn_decode_qkv");
 }

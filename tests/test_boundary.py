@@ -76,8 +76,9 @@ def test_argument_errors_return_before_any_launch(pkg):
     assert lib.scmx_gemv(C.byref(fmt), p, None, p, p, p, None, p, 1, 1, None, 0.0, 3, 8, 128, None, 0, 0, -1, None) == -1
     assert lib.scmx_quantize_sc(p, 0, 4, 96, 32, p, p, p, None) == -1                                 # K % (4 * block)
     assert lib.scmx_quantize_sc(p, 0, 4, 128, 24, p, p, p, None) == -1                                # block
-    assert lib.scmx_attn_decode(p, p, p, None, 5, p, 4, 2, 96, 64, 0.1, None) == -1                   # head dim
-    assert lib.scmx_attn_decode_qkv(p, p, p, 1e-6, p, None, 64, p, p, p, 4, 2, 128, 64, 0.1, None) == -1  # position outside the cache
+    assert lib.scmx_attn_decode(p, p, p, None, 5, p, 4, 2, 96, 64, 0.1, None, 1, None) == -1          # head dim
+    assert lib.scmx_attn_decode(p, p, p, None, 5, p, 4, 2, 128, 64, 0.1, None, 4, None) == -1         # splits without workspace
+    assert lib.scmx_attn_decode_qkv(p, p, p, 1e-6, p, None, 64, p, p, p, 4, 2, 128, 64, 0.1, None, 1, None) == -1  # position outside the cache
     assert lib.scmx_route_sort(p, 4, 8, 2000, 64, p, p, p, p, p, None) == -1                          # experts > 1024
     assert lib.scmx_mm_w4a8(C.byref(fmt), p, p, p, p, p, None, p, 1, 0, 8, 128, None) == 0            # M = 0: nothing to do
 

@@ -237,7 +237,7 @@ def test_fused_headnorm_rope_append_against_separate_ops(L, pos, from_acc):
         S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc, vc, rows - L + 1, inv_freq, **kw)
 
 
-@pytest.mark.parametrize("hq,hk,d,rows,n", [(16, 8, 128, 512, 129), (4, 4, 64, 40, 1), (8, 2, 256, 300, 300),
+@pytest.mark.parametrize("hq,hk,d,rows,n", [(16, 8, 128, 512, 129), (4, 4, 64, 40, 1), (8, 2, 256, 300, 300), (16, 8, 128, 8192, 5000),
                                             (16, 8, 128, 4096, 3000)])
 def test_attn_decode_against_torch(hq, hk, d, rows, n):
     from mxfp4_int8_m5_amd import sc_kernels as S
@@ -251,8 +251,12 @@ def test_attn_decode_against_torch(hq, hk, d, rows, n):
     ref = ref[0].transpose(0, 1).reshape(1, hq * d)
     o = S.attn_decode(q, kc, vc, n)
     assert o.shape == (1, hq * d) and rel(o, ref) < 6e-3, rel(o, ref)
-    o2 = S.attn_decode(q, kc, vc, torch.tensor([n - 1], device="cuda"))       # position from device memory
+    o2 = S.attn_decode(q, kc, vc, torch.tensor([n - 1], device="cuda"), splits=S.attn_splits(n))   # position from device memory
     assert torch.equal(o2, o)
+    for sp in (2, 7, 32):                                                      # rows cut into ranges, merged by a second kernel
+        o3 = S.attn_decode(q, kc, vc, n, splits=sp)
+        assert rel(o3, ref) < 6e-3 and rel(o3, o) < 3e-3, (sp, rel(o3, ref))
+        assert torch.equal(S.attn_decode(q, kc, vc, torch.tensor([n - 1], device="cuda"), splits=sp), o3)
     with pytest.raises(ValueError):
         S.attn_decode(q, kc, vc, rows + 1)
 
@@ -274,11 +278,13 @@ def test_attn_decode_qkv_equals_the_two_kernels(hq, hk, d, rows, pos):
     k1, v1, k2, v2, k3, v3 = kc.clone(), vc.clone(), kc.clone(), vc.clone(), kc.clone(), vc.clone()
     q = S.qkv_headnorm_rope(y, qn, kn, 1e-6, 1, hq, hk, d, k1, v1, pos, inv_freq)
     ref = S.attn_decode(q, k1, v1, pos + 1)
+    sp = S.attn_splits(pos + 1)                      # the same row ranges in every call: same summation order
+    assert sp == (1 if pos < 1024 else 16)
     out = S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k2, v2, pos, inv_freq)
     assert torch.equal(out, ref)
     assert torch.equal(k2, k1) and torch.equal(v2, v1)
     assert not torch.equal(k2[:, pos], kc[:, pos])                       # the row was written
-    out3 = S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k3, v3, torch.tensor([pos], device="cuda"), inv_freq)
+    out3 = S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k3, v3, torch.tensor([pos], device="cuda"), inv_freq, splits=sp)
     assert torch.equal(out3, ref) and torch.equal(k3, k1) and torch.equal(v3, v1)
     with pytest.raises(ValueError):
         S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k2, v2, rows, inv_freq)
