@@ -498,6 +498,22 @@ def main():
                 dec.step(ids[131 + j:132 + j], cache)
             torch.cuda.synchronize()
             model[name + "_tokens_per_s"] = round(32 / (time.perf_counter() - t0), 1)
+        # the same at a long context: 4000 cached tokens in a 4096-row cache (the decode attention then cuts the rows of a
+        # head into ranges; without that one workgroup per head would read 2 MB of K and V per block)
+        cache = fm.make_cache(4096)
+        long_ids = torch.randint(0, args.vocab_size, (4064,), device=dev, generator=g)
+        fm.hidden(long_ids[:2000], cache)
+        fm.hidden(long_ids[2000:4000], cache)
+        dec = FQ.DecodeQwen3(fm, graphs="step", fuse_prologue=True, head="packed")
+        for j in range(3):
+            dec.step(long_ids[4000 + j:4001 + j], cache)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for j in range(32):
+            dec.step(long_ids[4003 + j:4004 + j], cache)
+        torch.cuda.synchronize()
+        model["decode_graph_per_step_all_prologues_fused_packed_head_context_4000_tokens_per_s"] = round(
+            32 / (time.perf_counter() - t0), 1)
         del fm, dec, cache
         torch.cuda.empty_cache()
 
