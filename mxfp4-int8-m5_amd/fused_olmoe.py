@@ -23,6 +23,10 @@ from . import sc_moe
 from .fused_qwen3 import BF, KVCache, rms_norm
 from .sc_weights import PackedWeight
 
+# the reference keeps these two in its fused_olmoe module (e2e/fused_olmoe.py:74-97); the kernels live in sc_moe here
+moe_combine = sc_moe.moe_combine
+moe_combine_split = sc_moe.moe_combine_split
+
 ATTN = ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj"]   # e2e/fused_olmoe.py:28
 EXPERTS = ["gate_proj", "up_proj", "down_proj"]                                            # e2e/fused_olmoe.py:29
 
