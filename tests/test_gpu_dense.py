@@ -280,3 +280,42 @@ def test_config1_m8192_and_m512_equal_row_blocks_of_m2048(S, name, n, k):
         assert torch.equal(big[r0:r0 + 2048], S.linear_w4a8(x[r0:r0 + 2048].contiguous(), dc, db, dw, n)), (name, r0)
     for r0 in (0, 3584):
         assert torch.equal(big[r0:r0 + 512], S.linear_w4a8(x[r0:r0 + 512].contiguous(), dc, db, dw, n)), (name, r0)
+
+
+def test_random_shapes_formats_and_epilogues(S):
+    """Fifty seeded random problems (ragged M and N, K of 1 to 8 K steps, every test format, every epilogue) through
+    the dense GEMM, and row 0 of each through the GEMV: bit-exact against the oracle."""
+    from mxfp4_int8_m5_amd import sc_decode as G
+    rng = np.random.default_rng(2024)
+    done = 0
+    try:
+        while done < 50:
+            fmt = FORMATS[int(rng.integers(0, len(FORMATS)))]
+            m, n, k = int(rng.integers(1, 700)), int(rng.integers(1, 180)) * 4, int(rng.integers(1, 9)) * 128
+            if (k // fmt.block * fmt.bc_bits) % 8:
+                continue
+            pf = product_format(fmt)
+            S.set_format(pf)
+            codes, bc, ws, q = random_packed(rng, n, k, fmt)
+            xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+            xs = (np.abs(rng.standard_normal(m)) * 1e-2 + 1e-4).astype(F32)
+            epi = int(rng.integers(0, 4))
+            if epi == 3 and n % 8:
+                epi = 1
+            acc = linear.int_gemm(xq, q)
+            res = bf16.to_bits(rng.standard_normal((m, n)).astype(F32))
+            wq = S.unpack_i8(dev(codes), dev(bc), n, k)
+            if epi == 0:
+                got, want = host(S.mm_i8_i32(dev(xq), wq)), acc
+            else:
+                got = host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), epi, res=dev(res) if epi == 2 else None))
+                want = linear.epilogue(acc, xs, ws, epi, res if epi == 2 else None)
+            assert np.array_equal(got[:m], want), (done, fmt, m, n, k, epi)
+            ev = epi if epi else 1
+            y = host(G.gemv(dev(xq[0]), dev(codes), dev(bc), dev(xs[:1]), dev(ws), n, ev, res=dev(res[0]) if ev == 2 else None,
+                            fmt=pf))
+            wantv = linear.gemv(xq[0], xs[0], q, ws, ev, res[0] if ev == 2 else None)
+            assert np.array_equal(y.reshape(-1), np.asarray(wantv).reshape(-1)), (done, fmt, n, k, ev)
+            done += 1
+    finally:
+        S.set_format(product_format(layout.DEFAULT))
