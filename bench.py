@@ -498,6 +498,25 @@ def main():
                 dec.step(ids[131 + j:132 + j], cache)
             torch.cuda.synchronize()
             model[name + "_tokens_per_s"] = round(32 / (time.perf_counter() - t0), 1)
+        # the prefill attention kernel alone against the array library's op (2048 tokens, 16 / 8 heads of 128)
+        import torch.nn.functional as TF
+        from mxfp4_int8_m5_amd import sc_kernels as SK
+        qa = torch.randn(M_TOKENS, hq, d, device=dev, generator=g).to(torch.bfloat16)
+        ka = torch.randn(hk, M_TOKENS, d, device=dev, generator=g).to(torch.bfloat16)
+        va = torch.randn(hk, M_TOKENS, d, device=dev, generator=g).to(torch.bfloat16)
+        for label, fn in (("attn_prefill_us", lambda: SK.attn_prefill(qa.transpose(0, 1), ka, va, 0)),
+                          ("torch_attention_us", lambda: TF.scaled_dot_product_attention(
+                              qa.transpose(0, 1)[None], ka[None], va[None], is_causal=True, enable_gqa=True))):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for _ in range(20):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            model[label] = round(e0.elapsed_time(e1) / 20 * 1e3, 1)
+        del qa, ka, va
         # the same at a long context: 4000 cached tokens in a 4096-row cache (the decode attention then cuts the rows of a
         # head into ranges; without that one workgroup per head would read 2 MB of K and V per block)
         cache = fm.make_cache(4096)
