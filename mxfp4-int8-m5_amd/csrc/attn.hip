@@ -12,7 +12,7 @@
 
 namespace scmx {
 
-constexpr int ANT = 256;
+constexpr int ANT = 512;
 constexpr int ATTN_SINGLE_MAX = 512;   // rows up to which a split launch falls back to one workgroup per head
 
 // What the fused variant needs besides the attention operands: the token's q|k|v row as the qkv projection wrote it,

@@ -249,11 +249,11 @@ def qkv_headnorm_rope(y, qn, kn, eps, L, hq, hk, d, kcache, vcache, pos, inv_fre
 
 def attn_splits(rows):
     """Row ranges for the decode attention over up to `rows` cache rows: one workgroup per head reads a short context
-    fastest, longer ones are cut into 16 ranges (measured best from 1024 to 16000 rows: 9.6 / 11.2 / 20.7 / 41 us
-    at 1024 / 2048 / 4096 / 16000 rows against 23 / 43 / 86 / 354 us unsplit).  A split launch still serves
-    contexts of up to 512 rows with one workgroup per head (decided on the device), so a graph captured for a long
-    cache does not pay for the split while the context is short."""
-    return 1 if rows <= 1024 else 16
+    fastest, longer ones are cut into 8 ranges, beyond 8192 rows into 16 (measured: 8.6 / 10.2 / 16.3 / 34 us at
+    1024 / 2048 / 4096 / 16000 rows against 23 / 43 / 86 / 354 us unsplit).  A split launch still serves contexts of
+    up to 512 rows with one workgroup per head (decided on the device), so a graph captured for a long cache does not
+    pay for the split while the context is short."""
+    return 1 if rows <= 1024 else 8 if rows <= 8192 else 16
 
 
 def _split_workspace(splits, hq, d, device):

@@ -123,7 +123,7 @@ def test_attention_split_policy_and_cache_names(pkg):
     """Host-side choices that never touch the GPU: row ranges of the decode attention by context length, and the
     packed-cache file names of the reference (e2e/pack_format.py:79-80, e2e/fused_qwen3.py:331-333)."""
     S = pkg.sc_kernels
-    assert [S.attn_splits(n) for n in (1, 512, 1024, 1025, 4096, 100000)] == [1, 1, 1, 16, 16, 16]
+    assert [S.attn_splits(n) for n in (1, 512, 1024, 1025, 4096, 100000)] == [1, 1, 1, 8, 8, 16]
     from mxfp4_int8_m5_amd import pack_format as PF
     assert PF.cache_path("Qwen/Qwen3-1.7B", "e2m1/B16/M1..10", "/c") == "/c/Qwen--Qwen3-1.7B-fmt-e2m1_B16_M110.safetensors"
     f = PF.sc_format_of("e2m1/B16/M1..10")

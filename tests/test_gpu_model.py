@@ -279,7 +279,7 @@ def test_attn_decode_qkv_equals_the_two_kernels(hq, hk, d, rows, pos):
     q = S.qkv_headnorm_rope(y, qn, kn, 1e-6, 1, hq, hk, d, k1, v1, pos, inv_freq)
     ref = S.attn_decode(q, k1, v1, pos + 1)
     sp = S.attn_splits(pos + 1)                      # the same row ranges in every call: same summation order
-    assert sp == (1 if pos < 1024 else 16)
+    assert sp == (1 if pos < 1024 else 8)
     out = S.attn_decode_qkv(y, qn, kn, 1e-6, hq, hk, d, k2, v2, pos, inv_freq)
     assert torch.equal(out, ref)
     assert torch.equal(k2, k1) and torch.equal(v2, v1)
