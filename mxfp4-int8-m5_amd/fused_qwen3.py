@@ -214,9 +214,13 @@ class DecodeQwen3:
     (e2e/decode.py:29-99).  fuse_prologue="act" (default): RMSNorm + INT8 as separate kernels, the per-token INT8 of
     the o / down inputs inside those GEMVs' prologues; True: every quantization in a GEMV prologue; False: all
     separate.  graphs=True captures the two fixed-shape halves of every layer in HIP graphs on first use;
-    graphs="step" captures the whole step (all layers and the output head) as one graph per cache.  A graph is bound
-    to the cache it was captured with.  fuse_attn=True (default): q/k norm, rotary embedding, cache append and the
-    attention in one kernel; False: two kernels (same bits)."""
+    graphs="step" captures the whole step (all layers and the output head) as one graph per cache.  A graph holds raw
+    pointers into the cache it was captured with, so the decoder keeps that cache object alive next to the graph and
+    re-captures when it is handed a different one; `release(cache)` drops the graphs (and the reference) of a cache
+    that is no longer needed.  Tensors returned by `step` are fresh in every mode (the graphs' static outputs are
+    cloned).  fuse_attn=True (default): q/k norm, rotary embedding, cache append and the attention in one kernel;
+    False: two kernels (same bits).  head="packed": the output projection quantized to the published SC-MXFP4 format
+    (32-blocks, multipliers 1,2,4,8) whatever format the model's layers use."""
 
     def __init__(self, fused, fuse_prologue="act", graphs=False, head=True, fuse_attn=True):
         assert fused.epilogue == "gemm"
@@ -227,7 +231,8 @@ class DecodeQwen3:
         self.pos = torch.zeros(1, dtype=torch.int64, device=fused.device)   # position of the token being decoded
         self.packed_head = None
         if head == "packed":   # the output projection as SC-MXFP4 too (quantized here, on the device): 4x fewer bytes
-            codes, bc, ws, _ = F.quantize(fused.lm_head, None, with_q=False)
+            self.head_fmt = F.Format()          # named explicitly: independent of the process-wide default format
+            codes, bc, ws, _ = F.quantize(fused.lm_head, self.head_fmt, with_q=False)
             self.packed_head = (codes, bc, ws, fused.lm_head.shape[0])
 
     def _logits(self, h):
@@ -238,7 +243,7 @@ class DecodeQwen3:
         if self.packed_head is None:
             return f.logits(hn)
         codes, bc, ws, n = self.packed_head
-        return G.gemv(hn, codes, bc, None, ws, n, 1, pro=1)[None]
+        return G.gemv(hn, codes, bc, None, ws, n, 1, pro=1, fmt=self.head_fmt)[None]
 
     def _pre(self, h, nw, w, c, pos):
         f = self.f
@@ -280,9 +285,12 @@ class DecodeQwen3:
         xq, xs = S.act_quant(act[None], 1)
         return G.gemv(xq, wd.codes, wd.bcodes, xs, wd.wscale, wd.N, 2, res=h, fmt=f.fmt)[None]
 
-    def _capture(self, key, fn, inputs):
-        """Capture fn(*static copies of inputs) once per key; returns (graph, static inputs, static outputs)."""
-        if key not in self.graphs:
+    def _capture(self, key, fn, inputs, owner=None):
+        """Capture fn(*static copies of inputs) once per (key, owner); returns (graph, static inputs, static outputs).
+        `owner` is the object whose memory the captured kernels point into (a cache or one of its layers): it is stored
+        with the graph, which keeps it alive (its id cannot be reused by a later object), and an entry captured for a
+        different owner is replaced."""
+        if self._lookup(key, owner) is None:
             static = [t.clone() for t in inputs]
             s = torch.cuda.Stream()
             s.wait_stream(torch.cuda.current_stream())
@@ -292,15 +300,36 @@ class DecodeQwen3:
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 out = fn(*static)
-            self.graphs[key] = (g, static, out)
+            self.graphs[key] = (g, static, out, owner)
         return self.graphs[key]
 
-    def _replay(self, key, fn, inputs):
-        g, static, out = self._capture(key, fn, inputs)
+    def _lookup(self, key, owner):
+        """The entry stored under key if it was captured for this very owner object; an entry of another owner (a key
+        built from the id of an object that has since been replaced) is dropped."""
+        entry = self.graphs.get(key)
+        if entry is not None and entry[3] is not owner:
+            del self.graphs[key]
+            entry = None
+        return entry
+
+    def _replay(self, key, fn, inputs, owner=None):
+        g, static, out, _ = self._capture(key, fn, inputs, owner)
         for dst, src in zip(static, inputs):
             dst.copy_(src)
         g.replay()
         return out
+
+    def release(self, cache=None):
+        """Drop the captured graphs bound to `cache` (all graphs when None) together with the references that keep
+        their caches alive."""
+        if self.graphs is None:
+            return
+        if cache is None:
+            self.graphs.clear()
+            return
+        owners = [cache] + list(cache)
+        for key in [k for k, e in self.graphs.items() if any(e[3] is o for o in owners)]:
+            del self.graphs[key]
 
     # ---- the whole step as one HIP graph -----------------------------------------------------------------------
     # Everything that changes from token to token lives in device memory (token id, position): the fused
@@ -327,23 +356,24 @@ class DecodeQwen3:
         if self.graphs is not None:
             self.pos.fill_(off)
         if self.whole_step:
-            out = self._replay(("step", id(cache)), lambda t: self._step_static(t, cache), [tok])
+            out = self._replay(("step", id(cache)), lambda t: self._step_static(t, cache), [tok], owner=cache)
             for c in cache:
                 c.offset = off + 1
-            return out
+            return out.clone()     # the graph's static output is overwritten by the next replay
         h = f.embed[tok].contiguous()   # [1, D]
         for i, (nw, ws) in enumerate(f.layers):
             c = cache[i]
             if self.graphs is None:
                 q = self._pre(h, nw, ws["qkv"], c, off)
             else:
-                q = self._replay(("pre", i, id(c)), lambda x, nw=nw, w=ws["qkv"], c=c: self._pre(x, nw, w, c, self.pos), [h])
+                q = self._replay(("pre", i, id(c)), lambda x, nw=nw, w=ws["qkv"], c=c: self._pre(x, nw, w, c, self.pos), [h],
+                                 owner=c)
             o = self._attn(c, q)
             if self.graphs is None:
                 h = self._post(o, h, nw, ws)
             else:
                 h = self._replay(("post", i), lambda x, r, nw=nw, ws=ws: self._post(x, r, nw, ws), [o, h])
-        return self._logits(h)
+        return self._logits(h)      # new tensors: the final norm never returns a graph's static buffer
 
 
 # ---- from a checkpoint directory -----------------------------------------------------------------------------------

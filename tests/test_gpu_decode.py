@@ -193,3 +193,19 @@ def test_config2_lm_head_full_size(G, S):
     assert np.array_equal(y4, ref)
     y1 = host(G.gemv(dev(xb)[0], dc, db, None, dw, n, 1, pro=1))
     assert np.array_equal(y1, ref[0])
+
+
+@pytest.mark.parametrize("name,n,k", [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048),
+                                      ("down", 2048, 6144)])
+def test_config2_dense_shapes_full_size(G, name, n, k):
+    """BASELINE config 2 on the four dense layer shapes exactly as benchmarked: weights N(0, 0.02) quantized by the
+    oracle, a bf16 N(0, 1) token quantized in the kernel, batch 1 and batch 4; every output against the oracle."""
+    rng = np.random.default_rng(200 + n + k)
+    codes, bc, ws, q = layout.quantize(rng.standard_normal((n, k)) * 0.02)
+    xb = bf16.to_bits(rng.standard_normal((4, k)).astype(F32))
+    rq, rs = linear.act_quant(bf16.from_bits(xb))
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    ref = linear.gemv(rq, rs, q, ws, 1)
+    assert np.array_equal(host(G.gemv(dev(xb), dc, db, None, dw, n, 1, pro=1)), ref)
+    assert np.array_equal(host(G.gemv(dev(xb)[0], dc, db, None, dw, n, 1, pro=1)), ref[0])
+    assert linear.rel_fro(bf16.from_bits(ref[0]), linear.float_reference(bf16.from_bits(xb[:1]), q, ws)[0]) < 1e-2

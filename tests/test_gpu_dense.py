@@ -156,6 +156,31 @@ def test_config1_full_size_m2048(S, name, n, k):
     assert np.array_equal(host(S.mm_i8_i32(dev((a + b).astype(np.int8)), wq)), s)
 
 
+@pytest.mark.parametrize("name,n,k", [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048),
+                                      ("down", 2048, 6144)])
+def test_config1_quantized_weights_m2048(S, name, n, k):
+    """BASELINE config 1 at M = 2048 with weights generated as config 0 prescribes: N(0, 0.02) with 0.5 % of the input
+    columns scaled by 8, spread-constrained SC-MXFP4 quantization (the oracle's restatement of sim/make_testcase.py:
+    26-44), activations N(0, 1) with 1 % of the channels scaled by 20.  The one-call layer (quantization prologue +
+    fused-unpack GEMM + epilogue) bit for bit against the oracle, and within the north star's 1e-2 relative Frobenius
+    error of the float path (sim/make_testcase.py:59-60)."""
+    rng = np.random.default_rng(1000 + n + k)
+    m = 2048
+    w = llm_weights(rng, n, k)
+    codes, bc, ws, q = layout.quantize(w)
+    assert np.abs(q).max() <= 96
+    bits, x = llm_acts(rng, m, k)
+    xq_ref, xs_ref = linear.act_quant(x)
+    acc_ref = linear.int_gemm(xq_ref, q)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    y = host(S.linear_w4a8(dev(bits), dc, db, dw, n))
+    assert np.array_equal(y, linear.epilogue(acc_ref, xs_ref, ws, 1))
+    xq, xs = S.act_quant(dev(bits), Mp=m)
+    assert np.array_equal(host(S.mm_i8_i32(xq, S.unpack_i8(dc, db, n, k))), acc_ref)
+    assert linear.rel_fro(bf16.from_bits(y), linear.float_reference(x, q, ws)) < 1e-2   # the north star's tolerance
+    assert linear.rel_fro(bf16.from_bits(y), x.astype(np.float64) @ w.T) < 0.2
+
+
 def test_bad_arguments_raise(S):
     xq = torch.zeros((4, 100), dtype=torch.int8, device="cuda")
     wq = torch.zeros((8, 100), dtype=torch.int8, device="cuda")

@@ -173,6 +173,65 @@ def test_config3_olmoe_shape_property(M):
     assert np.array_equal(acc, moe.moe_int_gemm(xq, host(es), wq))
 
 
+def test_config3_pipeline_as_benchmarked(M):
+    """BASELINE config 3 at full size through the launches the benchmark times: 4096 tokens, 64 experts, top-8, hidden
+    2048, intermediate 1024, row tile 256: act_quant -> route_sort -> grouped gate|up GEMM reading token rows through
+    `gather` with the SwiGLU epilogue -> act_quant -> grouped down GEMM -> weighted combine (mirrors
+    e2e/fused_olmoe.py:207-245, checked like e2e/sc_moe.py:209-244).  The stages of the busiest, the emptiest non-empty
+    and a median expert bit for bit against the oracle; all 32768 rows independent of the row tile (64 vs 256); the
+    combine of all 4096 tokens against the oracle's sequential bf16 sum."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    rng = np.random.default_rng(3)
+    T, E, topk, D, Fi = 4096, 64, 8, 2048, 1024
+    R = T * topk
+    inds, scores = skewed_routing(rng, T, E, topk)
+    perm = linear.interleave_gate_up(Fi)
+    gu, dn = [], []
+    for _ in range(E):
+        c4 = rng.integers(0, 16, (2 * Fi, D), dtype=np.uint8)
+        b = rng.integers(0, 4, (2 * Fi, D // 32), dtype=np.uint8)
+        gu.append(layout.pack_rows(c4[perm], b[perm], np.exp2(rng.integers(-12, -6, 2 * Fi)).astype(F32)))
+        c4 = rng.integers(0, 16, (D, Fi), dtype=np.uint8)
+        b = rng.integers(0, 4, (D, Fi // 32), dtype=np.uint8)
+        dn.append(layout.pack_rows(c4, b, np.exp2(rng.integers(-12, -6, D)).astype(F32)))
+    gc, gb, gw = (dev(np.stack([p[i] for p in gu])) for i in range(3))
+    dc, db, dw = (dev(np.stack([p[i] for p in dn])) for i in range(3))
+    xb, x = llm_acts(rng, T, D)
+    res = bf16.to_bits(rng.standard_normal((T, D)).astype(F32))
+    xq, xs = S.act_quant(dev(xb), Mp=T)
+    outs = {}
+    for tm in (64, 256):
+        pos, tok, es, off, ts, mt = M.route_sort(dev(inds), E, tm)
+        moe.check_route_sort(inds, E, tm, host(pos), host(tok), host(es), host(off), host(ts))
+        act = M.moe_mm(xq, R, gc, gb, gw, off, ts, mt, 2 * Fi, 3, xs, tile=(tm, 64, 4), gather=tok)
+        aq, as_ = S.act_quant(act, Mp=R)
+        yd = M.moe_mm(aq, R, dc, db, dw, off, ts, mt, D, 1, as_, tile=(tm, 64, 4))
+        h, _, _ = M.moe_combine(yd, pos, dev(scores), dev(res), None, None, T, quant=False)
+        outs[tm] = (host(act)[host(pos)], host(yd)[host(pos)], host(h))
+    for a, b in zip(outs[64], outs[256]):
+        assert np.array_equal(a, b)
+    # the last pass is the benchmark's (row tile 256): its stages against the oracle on three experts
+    pos_h, off_h, tok_h = host(pos), host(off), host(tok)[:R]
+    counts = np.diff(off_h)
+    assert counts.sum() == R
+    rq, rs = linear.act_quant(x)
+    assert np.array_equal(host(xq), rq) and np.array_equal(host(xs), rs)
+    act_h, yd_h, aq_h, as_h = host(act), host(yd), host(aq), host(as_)
+    order = np.argsort(counts)
+    nonempty = order[counts[order] > 0]
+    for e in (int(nonempty[-1]), int(nonempty[0]), int(nonempty[len(nonempty) // 2])):
+        rows = slice(off_h[e], off_h[e + 1])
+        t = tok_h[rows]
+        q_gu = layout.decode(gu[e][0], gu[e][1], 2 * Fi, D)
+        a_ref = linear.epilogue(linear.int_gemm(rq[t], q_gu), rs[t], gu[e][2], 3)
+        assert np.array_equal(act_h[rows], a_ref), e
+        q2, s2 = linear.act_quant(bf16.from_bits(a_ref))
+        assert np.array_equal(aq_h[rows], q2) and np.array_equal(as_h[rows], s2), e
+        q_dn = layout.decode(dn[e][0], dn[e][1], D, Fi)
+        assert np.array_equal(yd_h[rows], linear.epilogue(linear.int_gemm(q2, q_dn), s2, dn[e][2], 1)), e
+    assert np.array_equal(outs[256][2], moe.combine(yd_h, pos_h, scores, res, T))
+
+
 def test_config4_sparse_moe_full_size(M):
     """BASELINE config 4 at its real shape: 256 routed experts + one shared expert (index 256), top-8 + shared = 9
     slots per token, hidden 2048, expert intermediate 512, the 16-element-block power-of-two format; 2048-token
