@@ -127,7 +127,8 @@ int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float*
 
 /* Single-token attention against a KV cache: out bf16 [hq * d] = softmax(q . K^T * scale) V per query head, q bf16
  * [hq, d], caches bf16 [hk, cache_rows, d] of which the first n rows are valid; n = *pos_dev + 1 when pos_dev != NULL
- * (device-resident position, for graph replay).  d in {64, 128, 256}.  Takes the place of the
+ * (device-resident position, for graph replay; a value outside 0 .. cache_rows - 1 gives an all-zero output and
+ * touches no cache row).  q and the caches 16-byte aligned.  d in {64, 128, 256}.  Takes the place of the
  * array library's scaled-dot-product attention at L = 1 in the decode step (e2e/decode.py:1-5, e2e/fused_qwen3.py:
  * 216-222), so that the step is a fixed launch sequence.  splits > 1 (at most 64; for long contexts): the valid rows
  * are cut into `splits` ranges, one workgroup per head and range, and a second launch merges the ranges' results out of
@@ -138,7 +139,8 @@ int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const uint16_t* 
 
 /* scmx_qkv_headnorm_rope at L = 1 and scmx_attn_decode in one launch: y bf16 [(hq + 2 hk) * d] is the token's q|k|v
  * row from the qkv projection; per-head RMSNorm of q and k, rotary embedding at position p (*pos_dev, or pos0 when
- * pos_dev is NULL), append of k and v to row p of the caches, attention over rows 0..p.  Same bits as the two calls
+ * pos_dev is NULL), append of k and v to row p of the caches, attention over rows 0..p (a device-resident p outside
+ * 0 .. cache_rows - 1 appends nothing and gives an all-zero output).  Same bits as the two calls
  * (with the same `splits`; workspace / splits as for scmx_attn_decode).
  * One launch less per block of the batch-1 decode step (e2e/decode.py:51-82; the array ops it stands for are
  * e2e/fused_qwen3.py:216-222). */
@@ -175,6 +177,17 @@ int scmx_gemv(const scmx_format* fmt, const void* x, const float* xscale, const 
               int shared_expert, void* stream);
 
 /* ---- mixture of experts ----------------------------------------------------------------------------------------- */
+
+/* Router: bf16 logits [M, n_experts] -> the topk experts of largest softmax probability per token and their scores.
+ * Probabilities are bf16(softmax in float32); scores are those probabilities, divided by their sum (bf16) when
+ * renorm != 0.  inds int32 / scores bf16 [M, topk], slots by falling probability, equal ones by rising expert index
+ * (the reference leaves both to argpartition).  shared_logit != NULL (bf16 [M], the shared expert's gate logit): one
+ * more slot per token, rows become [M, topk + 1] with inds = n_experts and score = bf16(sigmoid(shared_logit)).
+ * n_experts <= 1024, topk <= min(64, n_experts).  Replaces route, e2e/fused_olmoe.py:183-192 (softmax, argpartition,
+ * take_along_axis, optional renormalisation) and e2e/fused_qwen35.py:171-180 (renormalised, shared expert as the
+ * last slot with its sigmoid gate); the router's linear layer stays the caller's. */
+int scmx_route_topk(const uint16_t* logits, const uint16_t* shared_logit, int M, int n_experts, int topk, int renorm,
+                    int32_t* inds, uint16_t* scores, void* stream);
 
 /* Counting sort of the M*topk token-expert assignments by expert: pos [R], tok [R+tm], esorted [R], off [E+1],
  * tstart [E+1] (tile starts for row tiles of tm).  Replaces route_sort, e2e/sc_moe.py:114-155. */

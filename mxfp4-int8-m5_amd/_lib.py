@@ -39,6 +39,7 @@ SIGNATURES = {
     "scmx_qkv_headnorm_rope": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _L, _I, _I, _P]),
     "scmx_qkv_fullnorm": (_I, [_P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P]),
     "scmx_gemv": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _F, _I, _I, _I, _P, _I, _I, _I, _P]),
+    "scmx_route_topk": (_I, [_P, _P, _I, _I, _I, _I, _P, _P, _P]),
     "scmx_route_sort": (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P]),
     "scmx_moe_mm": (_I, [_FMT, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]),
     "scmx_moe_mm_i8": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]),

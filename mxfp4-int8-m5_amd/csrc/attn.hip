@@ -40,9 +40,17 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
     __shared__ float s_m[GROUPS], s_l[GROUPS], s_acc[GROUPS][D];
     __shared__ float s_sin[FUSED ? D / 2 : 1], s_cos[FUSED ? D / 2 : 1];
     __shared__ __attribute__((aligned(16))) uint16_t s_new[FUSED ? 3 : 1][D];   // this token's q, k, v (bf16)
-    const int n = min(rows, pos_dev ? int(pos_dev[0]) + 1 : n0);
     const int head = blockIdx.x, kvh = head / (hq / hk);
     const int tid = threadIdx.x, grp = tid / LPR, c = tid % LPR;
+    // A device-resident position outside the cache (the host cannot see it) touches no cache row: the output is
+    // zero and nothing is appended.
+    const int64_t n64 = pos_dev ? pos_dev[0] + 1 : int64_t(n0);
+    if (n64 < 1 || n64 > rows) {
+        if (blockIdx.y == 0)
+            for (int e = tid; e < D; e += ANT) out[size_t(head) * D + e] = 0;
+        return;
+    }
+    const int n = int(n64);
     const uint16_t* kbase = kc + size_t(kvh) * rows * D + 8 * c;
     const uint16_t* vbase = vc + size_t(kvh) * rows * D + 8 * c;
 
@@ -188,7 +196,8 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const uint16_t* __rest
 template <int D>
 __global__ __launch_bounds__(D) void attn_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out,
                                                      int splits, const int64_t* __restrict__ pos_dev, int n0, int rows) {
-    if (min(rows, pos_dev ? int(pos_dev[0]) + 1 : n0) <= ATTN_SINGLE_MAX) return;   // range 0 wrote the output itself
+    const int64_t n64 = pos_dev ? pos_dev[0] + 1 : int64_t(n0);
+    if (n64 <= ATTN_SINGLE_MAX || n64 > rows) return;   // range 0 wrote the output itself (zeros for a position outside the cache)
     const int head = blockIdx.x, e = threadIdx.x;
     const float* pw = partial + size_t(head) * splits * (D + 2);
     float mx = -3.0e38f;
@@ -251,6 +260,10 @@ extern "C" int scmx_attn_decode(const uint16_t* q, const uint16_t* kcache, const
         return SCMX_ERR_ARG;
     }
     if (int rc = check_attn("attn_decode", hq, hk, d, cache_rows)) return rc;
+    if (uintptr_t(q) % 16 || uintptr_t(kcache) % 16 || uintptr_t(vcache) % 16) {
+        set_error("attn_decode: q and the caches must be 16-byte aligned");
+        return SCMX_ERR_ARG;
+    }
     if (!pos_dev && (n < 1 || n > cache_rows)) {
         set_error("attn_decode: %d valid rows outside 1..%d", n, cache_rows);
         return SCMX_ERR_ARG;

@@ -465,6 +465,71 @@ static bool row_shape_ok(const char* who, int rows, int K, int max_k) {
     return true;
 }
 
+// ---- router: softmax over the experts, the k largest, renormalisation, shared-expert gate --------------------------
+// One wave per token.  Lane l holds experts l, l + 64, ...; probabilities are bf16(e_j / sum e) with
+// e_j = 1 / exp(min(max - x_j, 80)) (exp_pos: IEEE operations only, so a host restatement gives the same bits), the sum
+// taken per lane in rising j and then by the butterfly wave_sum.  The k winners are found by k wave-wide maxima over
+// the key (probability bits << 16 | 65535 - j): largest probability first, equal ones by rising expert index.
+constexpr int ROUTE_MAX_E = 1024;
+__global__ __launch_bounds__(NT) void route_topk_kernel(const uint16_t* __restrict__ logits,
+                                                        const uint16_t* __restrict__ shared_logit, int M, int E, int topk,
+                                                        int renorm, int32_t* __restrict__ inds,
+                                                        uint16_t* __restrict__ scores) {
+    constexpr int PER = ROUTE_MAX_E / 64;
+    const int lane = threadIdx.x & 63, t = blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+    if (t >= M) return;   // wave-uniform
+    const int stride = topk + (shared_logit ? 1 : 0);
+    const uint16_t* row = logits + size_t(t) * E;
+    float x[PER];
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+        const int j = 64 * c + lane;
+        x[c] = j < E ? bf16_to_f32(row[j]) : 0.0f;
+        if (j < E) mx = fmaxf(mx, x[c]);
+    }
+    mx = wave_max(mx);
+    float part = 0.0f;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+        const int j = 64 * c + lane;
+        x[c] = j < E ? __fdiv_rn(1.0f, exp_pos(fminf(__fsub_rn(mx, x[c]), 80.0f))) : 0.0f;
+        if (64 * c < E) part = __fadd_rn(part, x[c]);
+    }
+    const float total = wave_sum(part);
+    uint32_t key[PER];
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+        const int j = 64 * c + lane;
+        key[c] = j < E ? (uint32_t(f32_to_bf16(__fdiv_rn(x[c], total))) << 16) | uint32_t(0xFFFF - j) : 0u;
+    }
+    uint32_t mine = 0;      // lane s keeps the winner of round s
+    float tot = 0.0f;
+    for (int s = 0; s < topk; ++s) {
+        uint32_t best = 0;
+#pragma unroll
+        for (int c = 0; c < PER; ++c) best = max(best, key[c]);
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) best = max(best, uint32_t(__shfl_xor(int(best), off, WAVE)));
+#pragma unroll
+        for (int c = 0; c < PER; ++c)
+            if (key[c] == best) key[c] = 0;    // keys are distinct (they carry the expert index)
+        if (lane == s) mine = best;
+        tot = __fadd_rn(tot, bf16_to_f32(uint16_t(best >> 16)));
+    }
+    if (lane < topk) {
+        const uint16_t pb = uint16_t(mine >> 16);
+        inds[size_t(t) * stride + lane] = 0xFFFF - int(mine & 0xFFFFu);
+        scores[size_t(t) * stride + lane] = renorm ? f32_to_bf16(__fdiv_rn(bf16_to_f32(pb), round_bf16(tot))) : pb;
+    }
+    if (shared_logit && lane == 0) {
+        const float g = bf16_to_f32(shared_logit[t]);
+        const float y = __fdiv_rn(1.0f, __fadd_rn(1.0f, exp_pos(fminf(fabsf(g), 80.0f))));
+        inds[size_t(t) * stride + topk] = E;
+        scores[size_t(t) * stride + topk] = f32_to_bf16(g < 0.0f ? y : __fsub_rn(1.0f, y));
+    }
+}
+
 }  // namespace scmx
 
 using namespace scmx;
@@ -568,6 +633,20 @@ int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn,
     qkv_fullnorm_kernel<<<dim3(L), dim3(NT), size_t(h) * d * 2 + 72 * 4, (hipStream_t)stream>>>(y, qn, kn, eps, q, k, v, L,
                                                                                                  h, d);
     return check_launch("qkv_fullnorm");
+}
+
+int scmx_route_topk(const uint16_t* logits, const uint16_t* shared_logit, int M, int n_experts, int topk, int renorm,
+                    int32_t* inds, uint16_t* scores, void* stream) {
+    if (!logits || !inds || !scores || M < 0 || n_experts < 1 || n_experts > ROUTE_MAX_E || topk < 1 || topk > 64 ||
+        topk > n_experts) {
+        set_error("route_topk: null pointer, n_experts (%d) outside 1..%d or topk (%d) outside 1..min(64, n_experts)",
+                  n_experts, ROUTE_MAX_E, topk);
+        return SCMX_ERR_ARG;
+    }
+    if (M == 0) return SCMX_OK;
+    route_topk_kernel<<<dim3((M + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, (hipStream_t)stream>>>(
+        logits, shared_logit, M, n_experts, topk, renorm, inds, scores);
+    return check_launch("route_topk");
 }
 
 int scmx_route_sort(const int32_t* inds, int M, int topk, int n_experts, int tm, int32_t* pos, int32_t* tok,

@@ -6,7 +6,7 @@ Per transformer block (e2e/fused_olmoe.py:1-16):
   rope, KV cache, attention                                        torch ops (MLX ops in the reference)
   h = mm_epi(act_quant(o), Wo, + h)                                residual add in the GEMM epilogue
   xq, xs, xn = rmsnorm_quant_n(h)                                  INT8 for the experts, bf16 for the router
-  router: bf16 linear, float32 softmax, top-k                      torch ops
+  router: bf16 linear (torch), softmax + top-k (+ renorm) kernel   route
   route_sort; act = moe_mm(xq, gather=tok, Wg|Wu, SwiGLU)          token rows read through the sort, no xq[tok] copy
   y = moe_mm(act_quant(act), Wd); h, xq, xs = moe_combine(y, scores, + h) + next block's RMSNorm + INT8
 Expert weights stay packed; the grouped kernel decodes each expert's weight tile in LDS."""
@@ -127,13 +127,10 @@ class FusedOlmoe:
 
     def route(self, nw, xn, M):
         """mlx_lm's OlmoeSparseMoeBlock routing on the bf16 normalized rows (e2e/fused_olmoe.py:183-192): bf16 router
-        linear, float32 softmax, the k largest probabilities (their order within a token is irrelevant)."""
-        k = self.args.num_experts_per_tok
-        rw = torch.softmax((xn[:M] @ nw["mlp.gate"].T).float(), dim=1).to(BF)
-        scores, inds = torch.topk(rw, k, dim=-1, sorted=False)
-        if self.args.norm_topk_prob:
-            scores = scores / scores.sum(-1, keepdim=True)
-        return inds.to(torch.int32), scores.contiguous()
+        linear (an array op, as in the reference), then one kernel for the float32 softmax, the k largest probabilities
+        and the optional renormalisation."""
+        logits = xn[:M] @ nw["mlp.gate"].T
+        return sc_moe.route(logits, self.args.num_experts_per_tok, renorm=self.args.norm_topk_prob)
 
     def _experts(self, xq, xs, inds, scores, h, nn, ex, L, quant=True):
         a = self.args

@@ -13,6 +13,24 @@ from . import sc_format as F
 from . import sc_kernels as S
 
 
+def route(logits, k, renorm=True, shared_logit=None):
+    """Router on bf16 logits [M, E]: (inds int32 [M, k], scores bf16 [M, k]) = the k experts of largest softmax
+    probability (float32 softmax rounded to bf16) and their probabilities, divided by their sum when `renorm`
+    (e2e/fused_olmoe.py:183-192).  shared_logit bf16 [M]: a last slot with expert index E and score
+    sigmoid(shared_logit), outputs [M, k + 1] (e2e/fused_qwen35.py:171-180).  Slots are listed by falling probability."""
+    M, E = logits.shape
+    assert logits.dtype == torch.bfloat16 and (shared_logit is None or shared_logit.dtype == torch.bfloat16)
+    logits = logits.contiguous()
+    if shared_logit is not None:
+        shared_logit = shared_logit.reshape(M).contiguous()
+    width = k + (shared_logit is not None)
+    inds = torch.empty((M, width), dtype=torch.int32, device=logits.device)
+    scores = torch.empty((M, width), dtype=torch.bfloat16, device=logits.device)
+    _lib.call("scmx_route_topk", _lib.ptr(logits), _lib.ptr(shared_logit), M, E, k, int(bool(renorm)), _lib.ptr(inds),
+              _lib.ptr(scores), _lib.stream())
+    return inds, scores
+
+
 def route_sort(inds, n_experts, tm):
     """inds int [M, topk] -> (pos [R], tok [R + tm], e_sorted [R], off [E+1], tstart [E+1], max M-tiles)."""
     M, k = inds.shape

@@ -1,10 +1,55 @@
-"""Mixture-of-experts pieces (numpy; test infrastructure): the token sort / expert offsets, the grouped GEMM and
-the weighted combine."""
+"""Mixture-of-experts pieces (numpy; test infrastructure): the router (softmax, top-k, renormalisation, shared-expert
+gate), the token sort / expert offsets, the grouped GEMM and the weighted combine."""
 import numpy as np
 
 from . import bf16, linear
 
 F32 = np.float32
+
+
+def route(logit_bits, k, renorm=True, shared_bits=None):
+    """Router on bf16 logits [M, E] (uint16 bit patterns): probabilities = bf16(softmax in FP32), the k experts of
+    largest probability, their probabilities as scores, divided by their sum when `renorm` (every result rounded to
+    bf16, as array ops on bf16 arrays do) -> (inds int32 [M, k], score bits uint16 [M, k]).  With `shared_bits` (bf16
+    gate logits [M]) a last slot is appended: expert index E with score bf16(sigmoid(logit)).
+    Follows e2e/fused_olmoe.py:183-192 (softmax precise -> argpartition of the k largest -> take_along_axis ->
+    optional renormalisation) and e2e/fused_qwen35.py:171-180 (always renormalised, shared expert as slot k with its
+    sigmoid gate).  The reference leaves the order of the k slots and the choice among equal probabilities to
+    argpartition; this restatement lists them by falling probability, equal ones by rising expert index.
+    Arithmetic order (the one the device kernel uses): e_j = 1 / exp(min(max - x_j, 80)) with `linear.exp_f32`; the sum
+    of e over lane j % 64 in rising j, then the 64-lane butterfly of `linear._wave_sum`; p_j = bf16(e_j / sum); the
+    score total is the FP32 sum in slot order rounded to bf16.  Parity with the MLX ops themselves (softmax rounding at
+    a bf16 tie, argpartition's choice among equal probabilities) is unpinned; the restatement is pinned against torch
+    CPU ops and a brute-force top-k in tests/test_oracle_router.py."""
+    x = bf16.from_bits(np.asarray(logit_bits))
+    m, n_e = x.shape
+    d = np.minimum(x.max(1, keepdims=True) - x, F32(80.0)).astype(F32)
+    e = (F32(1.0) / linear.exp_f32(d)).astype(F32)
+    lanes = np.zeros((m, -(-n_e // 64) * 64), F32)
+    lanes[:, :n_e] = e
+    part = np.zeros((m, 64), F32)
+    for c in range(lanes.shape[1] // 64):          # lane l adds its experts l, l + 64, ... in rising order
+        part = part + lanes[:, 64 * c:64 * c + 64]
+    total = linear._wave_sum(part)
+    p_bits = bf16.to_bits((e / total[:, None]).astype(F32))
+    # k largest: key = probability bits (non-negative bf16 order like integers), ties to the lower index
+    key = p_bits.astype(np.int64) * 65536 + (65535 - np.arange(n_e, dtype=np.int64))[None, :]
+    inds = np.argsort(-key, axis=1, kind="stable")[:, :k].astype(np.int32)
+    s_bits = np.take_along_axis(p_bits, inds, 1)
+    if renorm:
+        s = bf16.from_bits(s_bits)
+        tot = np.zeros(m, F32)
+        for j in range(k):
+            tot = tot + s[:, j]
+        s_bits = bf16.to_bits((s / bf16.rnd(tot)[:, None]).astype(F32))
+    if shared_bits is not None:
+        g = bf16.from_bits(np.asarray(shared_bits).reshape(m))
+        ex = linear.exp_f32(np.minimum(np.abs(g), F32(80.0)))
+        y = (F32(1.0) / (F32(1.0) + ex)).astype(F32)
+        sig = np.where(g < 0, y, F32(1.0) - y).astype(F32)
+        inds = np.concatenate([inds, np.full((m, 1), n_e, np.int32)], 1)
+        s_bits = np.concatenate([s_bits, bf16.to_bits(sig)[:, None]], 1)
+    return inds, s_bits
 
 
 def route_sort(inds, n_experts, tm):

@@ -352,6 +352,54 @@ def test_packed_output_head(tiny):
     assert int(a.argmax()) == int(b.argmax()) or rel(b, a) < 0.1
 
 
+def test_packed_output_head_of_a_family_format_model(tiny, tmp_path):
+    """The packed head keeps the published format when the model's layers use another one (16-blocks, 4-bit block
+    codes), whether the decoder is built before or after the model's first pass selected its format."""
+    Q, args, state, packed = tiny
+    ckpt, cache_dir = str(tmp_path / "tiny-qwen3"), str(tmp_path / "cache")
+    _write_checkpoint(ckpt, args, state)
+    ids = torch.randint(0, args.vocab_size, (12,), generator=torch.Generator().manual_seed(8)).cuda()
+    m, _ = Q.load_fused(ckpt, cache_dir, packed="fmt:e2m1/B16/M1..10")
+    early = Q.DecodeQwen3(m, head="packed")                   # built before any pass set the model's format
+    c0, c1, c2 = m.make_cache(32), m.make_cache(32), m.make_cache(32)
+    for c in (c0, c1, c2):
+        m.hidden(ids[:11], c)
+    late = Q.DecodeQwen3(m, head="packed")                    # built after
+    a = Q.DecodeQwen3(m).step(ids[11:], c0)
+    b = early.step(ids[11:], c1)
+    c = late.step(ids[11:], c2)
+    assert torch.equal(b, c)
+    assert rel(b, a) < 0.15
+
+
+def test_one_decoder_over_successive_caches(tiny):
+    """A decoder with captured graphs used for one prompt after another, each with a cache of its own: every step equals
+    the eager decoder's on the same cache content, and graphs of a released cache are dropped."""
+    import gc
+    Q, args, state, packed = tiny
+    gen = torch.Generator().manual_seed(9)
+    m = Q.FusedQwen3(args, state, packed)
+    for graphs in (True, "step"):
+        dec, eager = Q.DecodeQwen3(m, graphs=graphs), Q.DecodeQwen3(m)
+        for prompt in range(4):
+            ids = torch.randint(0, args.vocab_size, (14,), generator=gen).cuda()
+            c1, c2 = m.make_cache(32), m.make_cache(32)
+            m.hidden(ids[:10], c1)
+            m.hidden(ids[:10], c2)
+            for j in range(10, 14):
+                a = eager.step(ids[j:j + 1], c1)
+                b = dec.step(ids[j:j + 1], c2)
+                torch.cuda.synchronize()
+                assert rel(b, a) < 1e-2, (graphs, prompt, j)
+            kept = b
+            if prompt % 2:
+                dec.release(c2)
+                assert not any(e[3] is c2 or any(e[3] is c for c in c2) for e in dec.graphs.values())
+            del c1, c2
+            gc.collect()
+        assert torch.equal(kept, b)            # returned logits are not aliased by later steps
+
+
 def _write_checkpoint(path, args, state):
     import dataclasses
     import json

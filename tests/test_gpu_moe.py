@@ -45,6 +45,36 @@ def test_route_sort_contract(M, m, topk, e, tm):
     assert np.array_equal(host(o2), ro[3]) and np.array_equal(host(t2), ro[4]) and mt2 == mt
 
 
+@pytest.mark.parametrize("m,e,k,renorm,shared", [(4096, 64, 8, True, False), (2048, 256, 8, True, True), (4096, 64, 8, False, False),
+                                                 (1, 64, 8, True, False), (77, 257, 9, True, False), (300, 1000, 64, False, True), (40, 1024, 3, True, False),
+                                                 (129, 8, 8, True, True), (50, 5, 1, True, False)])
+def test_router_against_oracle(M, m, e, k, renorm, shared):
+    """Softmax -> top-k -> renormalisation (-> shared-expert slot with its sigmoid gate) on config 3 / config 4 router
+    logits (N(0,1) + N(0,1.5) expert bias, bf16): expert indices and bf16 scores bit for bit against the oracle
+    (e2e/fused_olmoe.py:183-192, e2e/fused_qwen35.py:171-180)."""
+    rng = np.random.default_rng(m + e + k)
+    lb = bf16.to_bits((rng.standard_normal((m, e)) + rng.standard_normal(e) * 1.5).astype(F32))
+    if m > 4:
+        lb[1] = lb[1, 0]                      # a token with all-equal logits: ties resolved by rising index
+        lb[2, : e // 2] = lb[2, 0]
+    gl = bf16.to_bits((rng.standard_normal(m) * 3).astype(F32)) if shared else None
+    inds, scores = M.route(dev(lb), k, renorm=renorm, shared_logit=None if gl is None else dev(gl))
+    ri, rs = moe.route(lb, k, renorm, gl)
+    assert np.array_equal(host(inds), ri)
+    assert np.array_equal(host(scores), rs)
+    # and the result feeds the sort: every token's slots are distinct experts
+    pos, tok, es, off, ts, mt = M.route_sort(inds, e + int(shared), 64)
+    moe.check_route_sort(ri, e + int(shared), 64, host(pos), host(tok), host(es), host(off), host(ts))
+
+
+def test_router_bad_arguments(M):
+    lg = torch.zeros((4, 2000), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        M.route(lg, 8)                         # more than 1024 experts
+    with pytest.raises(ValueError):
+        M.route(lg[:, :4].contiguous(), 8)     # k > E
+
+
 @pytest.mark.parametrize("tm", [64, 128, 256])
 def test_grouped_gemm_uneven_segments(M, tm):
     """8 experts, 600 rows, experts 3 and 7 empty (e2e/sc_moe.py:213-215): INT32 exact, EPI 1 and 3 bit-exact,
