@@ -88,6 +88,19 @@ int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* 
                      const float* wscale, const uint16_t* res, void* out, int epi, int M, int N, int K,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* scmx_linear_w4a8 for callers that cannot allocate device memory or provide a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the INT8 activations and their scales are kept in a
+ * fixed array inside the library's device image instead of a workspace, so the call allocates nothing and takes no
+ * scratch argument.  No counterpart in the reference.  Limits: M * K <= scmx_linear_w4a8_static_max_elements()
+ * (16 Mi) and M <= scmx_linear_w4a8_static_max_rows() (16384); larger shapes return SCMX_ERR_WORKSPACE.  Same results as
+ * scmx_linear_w4a8.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
+ * or threads) race and must be serialised by the caller; each GPU holds 16.06 MiB for it until the process ends. */
+size_t scmx_linear_w4a8_static_max_elements(void);
+int scmx_linear_w4a8_static_max_rows(void);
+int scmx_linear_w4a8_static(const scmx_format* fmt, const uint16_t* x, const uint32_t* codes, const uint8_t* bcodes,
+                            const float* wscale, const uint16_t* res, void* out, int epi, int M, int N, int K,
+                            void* stream);
+
 /* ---- row kernels of the model integrations -------------------------------------------------------------------- */
 
 /* RMSNorm(x, w, eps) then per-token INT8; xn (optional, may be NULL) receives the normalized T rows [Mp, K].

@@ -29,6 +29,9 @@ SIGNATURES = {
     "scmx_mm_w4a8": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_linear_w4a8_workspace": (_Z, [_I, _I]),
     "scmx_linear_w4a8": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
+    "scmx_linear_w4a8_static_max_elements": (_Z, []),
+    "scmx_linear_w4a8_static_max_rows": (_I, []),
+    "scmx_linear_w4a8_static": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_rmsnorm_quant": (_I, [_P, _P, _F, _P, _P, _P, _I, _I, _I, _P]),
     "scmx_res_norm_quant": (_I, [_P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _P]),
     "scmx_swiglu_quant": (_I, [_P, _P, _P, _P, _P, _I, _I, _P]),

@@ -8,6 +8,7 @@
 // of 4 consecutive output columns n of one token row m, which is the unit every epilogue works on.
 // LDS holds three stages of the K loop; global loads run four steps ahead in two register sets, and the decode and
 // LDS writes of step i+2 are issued between the MFMAs of step i, with one barrier per step.
+#include <atomic>
 #include <type_traits>
 
 #include "scmx_common.h"
@@ -649,6 +650,64 @@ int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* 
     }
     int8_t* xq = reinterpret_cast<int8_t*>(workspace);
     float* xs = reinterpret_cast<float*>(xq + ((size_t(M) * size_t(K) + 255) & ~size_t(255)));
+    if (int rc = scmx_act_quant(x, xq, xs, M, M, K, stream)) return rc;
+    return scmx_mm_w4a8(fmt, xq, xs, codes, bcodes, wscale, res, out, epi, M, N, K, stream);
+}
+
+// ---- the dense layer for callers that cannot allocate ------------------------------------------------------------
+// The INT8 activations and their scales, which scmx_linear_w4a8 keeps in the caller's workspace, live here in a fixed
+// array of the library's device image (every GPU the library runs on holds its own copy until the process ends).
+// `scratch` is a host-side stand-in in host code, not a device address: the address on the current device comes from
+// hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+constexpr size_t STATIC_XQ_BYTES = size_t(16) << 20;   // M * K <= 16 Mi elements, e.g. 2048 x 8192 or 8192 x 2048
+constexpr int STATIC_MAX_ROWS = 16384;                 // M <= 16384 scales
+constexpr size_t STATIC_SCRATCH_BYTES = STATIC_XQ_BYTES + size_t(STATIC_MAX_ROWS) * sizeof(float);
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device (NULL with the error text set when it cannot be resolved).
+static uint8_t* static_scratch_device() {
+    static std::atomic<uint8_t*> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        set_error("linear_w4a8_static: no current device (or a device index beyond 63)");
+        return nullptr;
+    }
+    uint8_t* p = cached[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* addr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !addr) {
+            set_error("linear_w4a8_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        p = reinterpret_cast<uint8_t*>(addr);
+        cached[dev].store(p, std::memory_order_release);
+    }
+    return p;
+}
+
+size_t scmx_linear_w4a8_static_max_elements(void) { return STATIC_XQ_BYTES; }
+int scmx_linear_w4a8_static_max_rows(void) { return STATIC_MAX_ROWS; }
+
+int scmx_linear_w4a8_static(const scmx_format* fmt, const uint16_t* x, const uint32_t* codes, const uint8_t* bcodes,
+                            const float* wscale, const uint16_t* res, void* out, int epi, int M, int N, int K,
+                            void* stream) {
+    if (M < 0 || K <= 0) {
+        set_error("linear_w4a8_static: bad shape M=%d K=%d", M, K);
+        return SCMX_ERR_ARG;
+    }
+    if (size_t(M) * size_t(K) > STATIC_XQ_BYTES || M > STATIC_MAX_ROWS) {
+        set_error("linear_w4a8_static: M*K = %zu elements or M = %d rows beyond the built-in scratch (%zu elements, %d "
+                  "rows); use scmx_linear_w4a8 with a workspace", size_t(M) * size_t(K), M, STATIC_XQ_BYTES,
+                  STATIC_MAX_ROWS);
+        return SCMX_ERR_WORKSPACE;
+    }
+    uint8_t* base = static_scratch_device();
+    if (!base) return SCMX_ERR_LAUNCH;
+    int8_t* xq = reinterpret_cast<int8_t*>(base);
+    float* xs = reinterpret_cast<float*>(base + STATIC_XQ_BYTES);
+    // every byte of xq[M, K] and xs[M] that the GEMM reads is written by the quantization first: nothing has to start
+    // at zero, whatever the previous call left behind
     if (int rc = scmx_act_quant(x, xq, xs, M, M, K, stream)) return rc;
     return scmx_mm_w4a8(fmt, xq, xs, codes, bcodes, wscale, res, out, epi, M, N, K, stream);
 }
