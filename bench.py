@@ -1,13 +1,19 @@
 """Benchmark of the SC-MXFP4 W4A8 hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--reps R]
 
 One step = one pass of the dense W4A8 linear (activation-quantization prologue + fused-unpack INT8-MFMA GEMM + bf16
 epilogue, through the C ABI entry scmx_linear_w4a8) over the four Qwen3-1.7B-shaped layers at M = 2048 tokens
 (BASELINE config 1): qkv 4096x2048, o_proj 2048x2048, gate_up 12288x2048, down 2048x6144.  Inputs are seeded
 synthetic tensors already resident in HBM; weight sets rotate so that consecutive steps do not reuse cached weights.
-`value` is INT8 TOPS = 2*M*N*K summed over the layers / time.  The same run also reports the decode GEMV's achieved
-HBM GB/s (config 2) and a CPU baseline (the numpy oracle on the host cores).  Prints ONE JSON line.
+`value` is INT8 TOPS = 2*M*N*K summed over the layers / time.
+
+Timing protocol (the reference's, kernels/bench.swift:111-119 and e2e/bench_fused.py:71-91): every figure is taken
+after a warm-up of W steps and at least half a second of the same work, over R repetitions of K back-to-back steps,
+each repetition bracketed by events on the launch stream; the MEDIAN repetition is reported, the fastest one beside
+it.  The same run also reports the GEMM kernel alone (roofline), the step without its prologues, the decode GEMV's
+achieved HBM GB/s (config 2), the grouped expert passes (configs 3 and 4) and a CPU baseline (the numpy oracle on the
+host cores).  Prints ONE JSON line.
 """
 import argparse
 import ctypes as C
@@ -47,6 +53,32 @@ def acts(rng, m, k):
     return x
 
 
+def timed(torch, stream, fn, steps, reps=10, warmup=0, warm_s=0.5):
+    """fn(i) enqueues one step.  Warm up (`warmup` steps, then until `warm_s` seconds have passed), then time `reps`
+    repetitions of `steps` back-to-back steps, each between two events on `stream`.  Returns (median, min) ms per step."""
+    i = 0
+    for _ in range(warmup):
+        fn(i)
+        i += 1
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < warm_s:
+        for _ in range(max(1, min(steps, 16))):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    ev[0].record(stream)
+    for r in range(reps):
+        for _ in range(steps):
+            fn(i)
+            i += 1
+        ev[r + 1].record(stream)
+    torch.cuda.synchronize()
+    per = sorted(ev[r].elapsed_time(ev[r + 1]) / steps for r in range(reps))
+    return (per[reps // 2] if reps % 2 else 0.5 * (per[reps // 2 - 1] + per[reps // 2])), per[0]
+
+
 def cpu_baseline(budget_s=12.0):
     """The oracle's path (numpy): per-token INT8 quantization, float64-BLAS integer GEMM, FP32 scaling, bf16 rounding,
     for the four layers at M = 2048 with pre-decoded INT8 weights; repeated until the time budget is used."""
@@ -80,8 +112,9 @@ def cpu_baseline(budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--reps", type=int, default=10, help="timed repetitions of --steps steps (median reported)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV leg")
     ap.add_argument("--no-moe", action="store_true", help="skip the grouped mixture-of-experts leg")
@@ -146,51 +179,58 @@ def main():
         for args in calls[i % n_sets]:
             check(lib.scmx_linear_w4a8(*args))
 
-    for i in range(a.warmup):
-        run_step(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(a.steps):
-        run_step(i)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms_step = e0.elapsed_time(e1) / a.steps
+    timeit = lambda fn, steps, **kw: timed(torch, stream, fn, steps, **kw)   # noqa: E731
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)   # for the short side legs
+    ms_step, ms_step_min = timeit(run_step, a.steps, reps=a.reps, warmup=a.warmup)
     ops_step = sum(2.0 * M_TOKENS * n * k for _, n, k in LAYERS)
     tops = ops_step / (ms_step * 1e-3) / 1e12
+
+    # the same step without its prologues (activations quantized beforehand), and the prologues alone: where the
+    # difference between `value` and the GEMM kernel's rate goes
+    pre = {}
+    for k in xs_in:
+        xq = torch.empty((M_TOKENS, k), dtype=torch.int8, device=dev)
+        xs = torch.empty(M_TOKENS, dtype=torch.float32, device=dev)
+        check(lib.scmx_act_quant(xs_in[k].data_ptr(), xq.data_ptr(), xs.data_ptr(), M_TOKENS, M_TOKENS, k, sp))
+        pre[k] = (xq, xs)
+    gcalls = [[(C.byref(fmt), pre[k][0].data_ptr(), pre[k][1].data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(),
+                None, out.data_ptr(), 1, M_TOKENS, n, k, sp) for (name, n, k), (codes, bc, ws), out in zip(LAYERS, st, outs)]
+              for st in sets]
+
+    def run_gemms(i):
+        for args in gcalls[i % n_sets]:
+            check(lib.scmx_mm_w4a8(*args))
+
+    def run_prologues(i):
+        for _, _, k in LAYERS:
+            check(lib.scmx_act_quant(xs_in[k].data_ptr(), pre[k][0].data_ptr(), pre[k][1].data_ptr(), M_TOKENS, M_TOKENS,
+                                     k, sp))
+    ms_gemms, _ = timeit(run_gemms, a.steps, reps=a.reps, warm_s=0.3)
+    ms_pro, _ = timeit(run_prologues, a.steps, reps=a.reps, warm_s=0.2)
+    step_parts = {"step_ms": round(ms_step, 4), "step_ms_min": round(ms_step_min, 4),
+                  "gemms_only_ms": round(ms_gemms, 4), "gemms_only_tops": round(ops_step / ms_gemms / 1e9, 1),
+                  "prologues_only_ms": round(ms_pro, 4),
+                  "value_over_gemms_only": round(ms_gemms / ms_step, 3),
+                  "note": "4 layers per step; gemms_only = the four scmx_mm_w4a8 launches back to back on pre-quantized "
+                          "activations; prologues_only = the four scmx_act_quant launches"}
 
     # ---- roofline of the dominant kernel (the fused-unpack GEMM alone, activations pre-quantized) -------------------
     per_shape = {}
     tot_ops = tot_ms = 0.0
-    reps = max(20, a.steps // 2)
     for li, (name, n, k) in enumerate(LAYERS):
-        xq = torch.empty((M_TOKENS, k), dtype=torch.int8, device=dev)
-        xs = torch.empty(M_TOKENS, dtype=torch.float32, device=dev)
-        check(lib.scmx_act_quant(xs_in[k].data_ptr(), xq.data_ptr(), xs.data_ptr(), M_TOKENS, M_TOKENS, k, sp))
-        argl = []
-        for s in sets:
-            codes, bc, ws = s[li]
-            argl.append((C.byref(fmt), xq.data_ptr(), xs.data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(), None,
-                         outs[li].data_ptr(), 1, M_TOKENS, n, k, sp))
-        for i in range(5):
-            check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
-        torch.cuda.synchronize()
-        e0.record(stream)
-        for i in range(reps):
-            check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
-        e1.record(stream)
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps
+        argl = [g[li] for g in gcalls]
+        ms, ms_min = timeit(lambda i: check(lib.scmx_mm_w4a8(*argl[i % n_sets])), max(20, a.steps), reps=a.reps, warm_s=0.5)
         ops = 2.0 * M_TOKENS * n * k
-        per_shape[name] = {"us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
+        per_shape[name] = {"us": round(ms * 1e3, 2), "us_min": round(ms_min * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
                            "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
         tot_ops += ops
         tot_ms += ms
     achieved = tot_ops / tot_ms / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": GEMM_TRAFFIC_BYTES, "kernel": "scmx::gemm_kernel (mm_w4a8)",
-                "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their average launch "
-                        "durations, activations pre-quantized", "per_shape": per_shape}
+                "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their launch durations "
+                        "(median repetition of back-to-back launches between events on the launch stream), "
+                        "activations pre-quantized", "per_shape": per_shape}
 
     # ---- the ROCm library's INT8 GEMM on the same shapes: what tuned vendor code reaches here with resident INT8 ----
     # weights, INT32 output, no unpack and no epilogue (a reference point for the fraction of peak, not a baseline)
@@ -200,15 +240,7 @@ def main():
             for name, n, k in LAYERS:
                 xa = torch.randint(-127, 128, (M_TOKENS, k), dtype=torch.int8, device=dev)
                 wb = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev).t()
-                for _ in range(3):
-                    torch._int_mm(xa, wb)
-                torch.cuda.synchronize()
-                e0.record(stream)
-                for _ in range(20):
-                    torch._int_mm(xa, wb)
-                e1.record(stream)
-                torch.cuda.synchronize()
-                ms = e0.elapsed_time(e1) / 20
+                ms, _ = timeit(lambda i: torch._int_mm(xa, wb), 20, reps=5, warm_s=0.2)
                 library[name] = {"us": round(ms * 1e3, 2), "tops": round(2.0 * M_TOKENS * n * k / ms / 1e9, 1)}
                 del xa, wb
             library["what"] = "torch._int_mm at M = %d: INT8 x INT8 -> INT32, weights already INT8, no epilogue" % M_TOKENS
@@ -230,16 +262,7 @@ def main():
                     codes, bc, ws = s[li]
                     argl.append((C.byref(fmt), xq.data_ptr(), xs.data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(),
                                  None, out.data_ptr(), 1, m, n, k, sp))
-                for i in range(10):   # long enough for the clocks to settle after the host-side preparation
-                    check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
-                torch.cuda.synchronize()
-                reps_s = 40
-                e0.record(stream)
-                for i in range(reps_s):
-                    check(lib.scmx_mm_w4a8(*argl[i % n_sets]))
-                e1.record(stream)
-                torch.cuda.synchronize()
-                ms = e0.elapsed_time(e1) / reps_s
+                ms, _ = timeit(lambda i: check(lib.scmx_mm_w4a8(*argl[i % n_sets])), 20, reps=a.reps, warm_s=0.3)
                 ops = 2.0 * m * n * k
                 sweep[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
                                          "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
@@ -252,10 +275,7 @@ def main():
         T, E, TOPK, D, Fi, TM = 4096, 64, 8, 2048, 1024, int(os.environ.get('SCMX_BENCH_TM', '256'))
         R = T * TOPK
         logits = rng.standard_normal((T, E)) + rng.standard_normal(E) * 1.5      # biased router: skewed expert loads
-        inds_np = np.argsort(-logits, axis=1)[:, :TOPK]
-        p = np.exp(np.take_along_axis(logits, inds_np, 1))
-        scores = up((p / p.sum(1, keepdims=True)).astype(np.float32)).to(torch.bfloat16)
-        inds = up(inds_np.astype(np.int32))
+        logits_d = up(logits.astype(np.float32)).to(torch.bfloat16)              # router logits, resident
         x = up(acts(rng, T, D)).to(torch.bfloat16)
 
         def experts(n, k):
@@ -266,28 +286,20 @@ def main():
 
         def moe_pass():
             xq, xs = SK.act_quant(x, T)
+            inds, scores = SM.route(logits_d, TOPK, renorm=True)
             pos, tok, _, off, tstart, mt = SM.route_sort(inds, E, TM)
             h = SM.moe_mm(xq, R, gu[0], gu[1], gu[2], off, tstart, mt, 2 * Fi, 3, xscale=xs, tile=(TM, 64, 4), gather=tok)
             hq, hs = SK.act_quant(h, R)
             y = SM.moe_mm(hq, R, dn[0], dn[1], dn[2], off, tstart, mt, D, 1, xscale=hs, tile=(TM, 64, 4))
             return SM.moe_combine(y, pos, scores, x, None, 0.0, T, quant=False)[0]
 
-        for _ in range(3):
-            moe_pass()
-        torch.cuda.synchronize()
-        reps_m = 20
-        e0.record(stream)
-        for _ in range(reps_m):
-            moe_pass()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps_m
-        tiles = int(SM.route_sort(inds, E, TM)[4][-1].item())
+        ms, ms_min3 = timeit(lambda i: moe_pass(), 10, reps=a.reps, warm_s=0.3)
+        tiles = int(SM.route_sort(SM.route(logits_d, TOPK)[0], E, TM)[4][-1].item())
         ops = 2.0 * R * 3 * Fi * D
-        moe = {"workload": "BASELINE configs[3]: act quant + token sort + grouped gate_up GEMM (SwiGLU epilogue) + act "
+        moe = {"workload": "BASELINE configs[3]: act quant + router (softmax, top-8, renormalisation) + token sort + grouped gate_up GEMM (SwiGLU epilogue) + act "
                            "quant + grouped down GEMM + weighted combine", "tokens": T, "experts": E, "topk": TOPK,
                "row_tile": TM, "row_tiles": tiles, "padded_rows_pct": round((tiles * TM / R - 1) * 100, 1),
-               "ms": round(ms, 4), "tops": round(ops / ms / 1e9, 1),
+               "ms": round(ms, 4), "ms_min": round(ms_min3, 4), "tops": round(ops / ms / 1e9, 1),
                "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
         del gu, dn, x
         torch.cuda.empty_cache()
@@ -306,27 +318,21 @@ def main():
                     torch.full((E4, n), 2.0 ** -9, dtype=torch.float32, device=dev))
         gu4, dn4 = experts16(2 * F4, D4), experts16(D4, F4)
         lg = rng.standard_normal((T4, E4 - 1)) + rng.standard_normal(E4 - 1) * 1.5
-        top = np.argsort(-lg, axis=1)[:, :8]
-        inds4 = up(np.concatenate([top, np.full((T4, 1), E4 - 1)], 1).astype(np.int32))
+        lg_d = up(lg.astype(np.float32)).to(torch.bfloat16)
+        sg_d = up(rng.standard_normal(T4).astype(np.float32)).to(torch.bfloat16)    # the shared expert's gate logits
+        inds4 = SM.route(lg_d, 8, renorm=True, shared_logit=sg_d)[0]                 # [T4, 9]: top-8 + the shared slot
         x4 = up(acts(rng, T4, D4)).to(torch.bfloat16)
 
         def pass4():
             xq, xs = SK.act_quant(x4, T4)
-            pos, tok, _, off, tstart, mt = SM.route_sort(inds4, E4, TM4)
+            inds9, _ = SM.route(lg_d, 8, renorm=True, shared_logit=sg_d)
+            pos, tok, _, off, tstart, mt = SM.route_sort(inds9, E4, TM4)
             h = SM.moe_mm(xq, R4, gu4[0], gu4[1], gu4[2], off, tstart, mt, 2 * F4, 3, xscale=xs, tile=(TM4, 64, 4),
                           gather=tok, fmt=f16)
             hq, hs = SK.act_quant(h, R4)
             return SM.moe_mm(hq, R4, dn4[0], dn4[1], dn4[2], off, tstart, mt, D4, 1, xscale=hs, tile=(TM4, 64, 4), fmt=f16)
 
-        for _ in range(3):
-            pass4()
-        torch.cuda.synchronize()
-        e0.record(stream)
-        for _ in range(20):
-            pass4()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        ms4 = e0.elapsed_time(e1) / 20
+        ms4, ms4_min = timeit(lambda i: pass4(), 10, reps=a.reps, warm_s=0.3)
         # batch-1 decode: the 9-slot gate|up and down GEMVs of one token, replayed from a HIP graph
         xq1, xs1 = SK.act_quant(x4[:1].contiguous(), 1)
         eidx = inds4[0, :8].contiguous()
@@ -353,10 +359,16 @@ def main():
         us_tok = e0.elapsed_time(e1) / 100 * 1e3
         bytes_tok = 9 * 3 * F4 * D4 * (0.5 + 1.0 / 64)
         ops4 = 2.0 * R4 * 3 * F4 * D4
+        # config 4's prefill streams every expert's weights once for ~72 rows each: 278 op/B, below the ~630 op/B ridge,
+        # so its roof is HBM: packed expert weights + bf16 tokens in + bf16 rows out
+        bytes4 = E4 * 3 * F4 * D4 * (0.5 + 1.0 / 64) + 2.0 * T4 * D4 + 2.0 * R4 * D4
         moe["config4"] = {"workload": "BASELINE configs[4]: 257 experts (256 routed + shared), 9 slots per token, 16-block "
-                                      "format; prefill of 2048 tokens (act quant, sort, two grouped GEMMs, act quant) and "
+                                      "format; prefill of 2048 tokens (act quant, router with the shared slot, sort, two grouped GEMMs, act quant) and "
                                       "the two 9-slot GEMVs of one decode token",
-                          "prefill_ms": round(ms4, 4), "prefill_tops": round(ops4 / ms4 / 1e9, 1), "row_tile": TM4,
+                          "prefill_ms": round(ms4, 4), "prefill_ms_min": round(ms4_min, 4),
+                          "prefill_tops": round(ops4 / ms4 / 1e9, 1), "prefill_bound": "hbm",
+                          "prefill_gbps": round(bytes4 / ms4 / 1e6, 1),
+                          "prefill_pct_hbm": round(bytes4 / ms4 / 1e6 / PEAK_HBM_GBPS * 100, 1), "row_tile": TM4,
                           "decode_us_per_token": round(us_tok, 2), "decode_gbps": round(bytes_tok / us_tok / 1e3, 1)}
         del gu4, dn4, graph
         torch.cuda.empty_cache()
@@ -376,19 +388,29 @@ def main():
                 out = torch.empty((batch, n), dtype=torch.bfloat16, device=dev)
                 argl = [(C.byref(fmt), x.data_ptr(), None, c.data_ptr(), b.data_ptr(), w.data_ptr(), None, out.data_ptr(),
                          1, 1, None, C.c_float(0.0), batch, n, k, None, 0, 0, -1, sp) for c, b, w in wsets]
-                for i in range(copies):
-                    check(lib.scmx_gemv(*argl[i]))
-                torch.cuda.synchronize()
                 reps_d = max(copies, 100)
-                e0.record(stream)
-                for i in range(reps_d):
-                    check(lib.scmx_gemv(*argl[i % copies]))
-                e1.record(stream)
-                torch.cuda.synchronize()
-                us = e0.elapsed_time(e1) / reps_d * 1e3
+                ms_d, ms_d_min = timeit(lambda i: check(lib.scmx_gemv(*argl[i % copies])), reps_d, reps=a.reps, warmup=copies,
+                                   warm_s=0.2)
+                us = ms_d * 1e3
+                # the same launches replayed from a HIP graph: kernel time without the host's per-call launch cost
+                ncap = min(copies, 40)
+                side = torch.cuda.Stream()
+                side.wait_stream(stream)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    ssp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                    for i in range(ncap):
+                        check(lib.scmx_gemv(*(argl[i][:-1] + (ssp,))))
+                stream.wait_stream(side)
+                ms_g, _ = timeit(lambda i: graph.replay(), max(2, 100 // ncap), reps=a.reps, warm_s=0.1)
+                us_g = ms_g * 1e3 / ncap
                 bts = n * k * (0.5 + 1.0 / 128) + 4 * n + batch * (2 * k + 2 * n)
-                decode[f"{name}_b{batch}"] = {"us": round(us, 2), "gbps": round(bts / us / 1e3, 1),
-                                              "pct_hbm": round(bts / us / 1e3 / PEAK_HBM_GBPS * 100, 1)}
+                decode[f"{name}_b{batch}"] = {"us": round(us, 2), "us_min": round(ms_d_min * 1e3, 2),
+                                              "gbps": round(bts / us / 1e3, 1),
+                                              "pct_hbm": round(bts / us / 1e3 / PEAK_HBM_GBPS * 100, 1),
+                                              "us_graph": round(us_g, 2), "gbps_graph": round(bts / us_g / 1e3, 1),
+                                              "pct_hbm_graph": round(bts / us_g / 1e3 / PEAK_HBM_GBPS * 100, 1)}
+                del graph
             del wsets
             torch.cuda.empty_cache()
 
@@ -539,12 +561,19 @@ def main():
     result = {
         "metric": "INT8 TOPS, W4A8 prefill GEMM M=2048 (Qwen3-1.7B layer shapes), 1 GPU; decode GEMV GB/s alongside",
         "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_step, 4), "ms_per_step_min": round(ms_step_min, 4), "repetitions": a.reps,
+        "timing": "median of `repetitions` repetitions of `steps` back-to-back steps after `warmup` steps + 0.5 s of warm-up",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "BASELINE configs[1] at M=2048: SC-MXFP4 W4A8 linear (act-quant prologue + fused-unpack "
                                "INT8 MFMA GEMM + bf16 epilogue) over qkv 4096x2048, o_proj 2048x2048, gate_up 12288x2048, "
                                "down 2048x6144", "tokens": M_TOKENS, "weight_sets_rotated": n_sets},
         "pct_int8_peak": round(tops / PEAK_INT8_TOPS * 100, 2),
+        "system": {"library": lib.scmx_version().decode(), "torch": torch.__version__, "rocm": torch.version.hip,
+                   "device": torch.cuda.get_device_name(0),
+                   "compute_units": torch.cuda.get_device_properties(0).multi_processor_count,
+                   "host_cores": os.cpu_count()},
+        "step_parts": step_parts,
         "roofline": roofline,
         "prefill_sweep": sweep,
         "library_int8_gemm": library,

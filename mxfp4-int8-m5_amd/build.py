@@ -22,12 +22,29 @@ def _run(cmd):
     return out
 
 
+def _build_id():
+    """Source revision for scmx_version(): the git commit of the tree (with "+" when files differ from it), or "unknown"
+    outside a checkout."""
+    try:
+        root = os.path.dirname(HERE)
+        rev = subprocess.run(["git", "-C", root, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True, timeout=20)
+        if rev.returncode:
+            return "unknown"
+        dirty = subprocess.run(["git", "-C", root, "status", "--porcelain", "--untracked-files=no"], capture_output=True,
+                               text=True, timeout=20).stdout.strip()
+        return rev.stdout.strip() + ("+" if dirty else "")
+    except Exception:
+        return "unknown"
+
+
 def build(verbose=False):
     hipcc = os.environ.get("HIPCC", "hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
-    cmds = [[hipcc, *FLAGS, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
+    bid = ['-DSCMX_BUILD_ID="%s"' % _build_id()]
+    cmds = [[hipcc, *FLAGS, *(bid if s == "api.hip" else []), "-c", os.path.join(CSRC, s), "-o", o]
+            for s, o in zip(SOURCES, objs)]
     with ThreadPoolExecutor(4) as ex:
         for out in ex.map(_run, cmds):
             if verbose and out.strip():

@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "scmx_common.h"
 
 namespace scmx {
@@ -24,6 +26,19 @@ int check_launch(const char* what) {
         return SCMX_ERR_LAUNCH;
     }
     return SCMX_OK;
+}
+
+// Compute units of the current device, asked once per device (256 on MI355X; the fallback when the query fails).
+int device_cus() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
 }
 
 int make_dev_format(const scmx_format* f, DevFormat* out) {
@@ -301,7 +316,11 @@ using namespace scmx;
 
 extern "C" {
 
-const char* scmx_version(void) { return "scmx 0.1 (gfx950)"; }
+#ifndef SCMX_BUILD_ID
+#define SCMX_BUILD_ID "unknown"
+#endif
+// "scmx <version> (gfx950) <source revision the library was built from>"
+const char* scmx_version(void) { return "scmx 0.2 (gfx950) " SCMX_BUILD_ID; }
 const char* scmx_last_error(void) { return g_err; }
 
 void scmx_default_format(scmx_format* f) {

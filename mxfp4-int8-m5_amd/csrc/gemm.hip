@@ -539,9 +539,9 @@ static int packed_mode(const DevFormat& f) {
 // Dense: the largest tile that still gives every CU a workgroup.  256x256 (wave tiles of 128x64, K steps of 64) moves
 // 25 % fewer LDS bytes per MFMA than 256x128 and is worth 4-5 % where the problem has 256 such tiles.
 static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
-    const long cus = 256;
+    const long cus = device_cus();
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-    // the widest tile only where its tiles fill whole rounds of the 256 CUs (a last round that is mostly empty costs
+    // the widest tile only where its tiles fill whole rounds of the CUs (a last round that is mostly empty costs
     // more than the narrower tile's extra LDS traffic: 384 tiles would take 2 rounds of double-size work)
     const long t256 = tiles(256, 256);
     if (t256 >= cus && t256 * 100 >= ((t256 + cus - 1) / cus) * cus * 88)

@@ -52,6 +52,9 @@ inline bool is_block16_range_format(const DevFormat& d) {
     return m0 >= 1;
 }
 
+// Compute units of the current device (queried once per device).
+int device_cus();
+
 // Thread-local error text behind scmx_last_error().
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
