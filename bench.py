@@ -308,7 +308,7 @@ def main():
         # 16-element-block power-of-two format; random code words (the kernels' time does not depend on the values)
         from mxfp4_int8_m5_amd import sc_decode as SD, sc_format as SF
         f16 = SF.Format(block=16)
-        T4, E4, D4, F4, TM4 = 2048, 257, 2048, 512, 64
+        T4, E4, D4, F4, TM4 = 2048, 257, 2048, 512, int(os.environ.get('SCMX_BENCH_TM4', '64'))
         R4 = T4 * 9
         gen = torch.Generator(device=dev).manual_seed(4)
 

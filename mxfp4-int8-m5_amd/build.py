@@ -53,5 +53,26 @@ def build(verbose=False):
     return LIB
 
 
+def build_host_check(driver, out=None):
+    """The library's sources and a C++ driver of the C ABI as ONE executable whose HOST code is instrumented with
+    AddressSanitizer and UBSan (device code is compiled as usual and never runs in this check): for machines without a
+    GPU, where every entry point ends at its argument checks or at the failing launch.  Returns the executable's path."""
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    objdir = os.path.join(HERE, "build", "host_check")
+    os.makedirs(objdir, exist_ok=True)
+    out = out or os.path.join(objdir, "boundary_check")
+    san = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-Xarch_host",
+           "-fno-sanitize-recover=undefined", "-g", "-fno-omit-frame-pointer"]
+    flags = [f for f in FLAGS if f != "-O3"] + ["-O1"]
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+    cmds = [[hipcc, *flags, *san, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
+    dobj = os.path.join(objdir, "driver.o")
+    cmds.append([hipcc, "-x", "hip", *flags, *san, "-c", driver, "-o", dobj])
+    with ThreadPoolExecutor(4) as ex:
+        list(ex.map(_run, cmds))
+    _run([hipcc, "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined", "-o", out, dobj, *objs])
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))

@@ -342,6 +342,10 @@ int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t*
                   (long long)K, f.block);
         return SCMX_ERR_ARG;
     }
+    if (K > (int64_t(1) << 30) || n_rows > (int64_t(1) << 40) / K) {   // keeps every count below 2^40 and the grid below 2^32
+        set_error("unpack_i8: %lld x %lld weights are more than one launch takes (2^40)", (long long)n_rows, (long long)K);
+        return SCMX_ERR_ARG;
+    }
     if (n_rows == 0) return SCMX_OK;
     const int bc_row_bytes = int(K / f.block * f.bc_bits / 8);
     hipStream_t s = (hipStream_t)stream;
@@ -362,8 +366,8 @@ int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t*
 }
 
 int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream) {
-    if (!x || !xq || !xs || M < 0 || Mp < M || K <= 0 || K % 8 || uintptr_t(x) % 16 || uintptr_t(xq) % 8) {
-        set_error("act_quant: need M <= Mp, K %% 8 == 0 (K = %d), x 16-byte and xq 8-byte aligned", K);
+    if (!x || !xq || !xs || M < 0 || Mp < M || Mp > (1 << 30) || K <= 0 || K % 8 || uintptr_t(x) % 16 || uintptr_t(xq) % 8) {
+        set_error("act_quant: need M <= Mp <= 2^30, K %% 8 == 0 (K = %d), x 16-byte and xq 8-byte aligned", K);
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
@@ -399,8 +403,8 @@ int scmx_rot_quant(const uint16_t* x, const float* signs, int8_t* xq, float* xs,
 
 int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,
                      void* stream) {
-    if (!e8m0 || !bcodes || !wscale || !status || N < 0 || K <= 0 || K % 128) {
-        set_error("mxfp4_to_sc: need non-null pointers and K %% 128 == 0 (K = %lld)", (long long)K);
+    if (!e8m0 || !bcodes || !wscale || !status || N < 0 || N > (int64_t(1) << 32) || K <= 0 || K % 128 || K > (int64_t(1) << 30)) {
+        set_error("mxfp4_to_sc: need non-null pointers, N <= 2^32 and K %% 128 == 0, K <= 2^30 (K = %lld)", (long long)K);
         return SCMX_ERR_ARG;
     }
     if (N == 0) return SCMX_OK;

@@ -241,7 +241,7 @@ static int check_split(const char* who, const float* workspace, int splits) {
 using namespace scmx;
 
 static int check_attn(const char* who, int hq, int hk, int d, int cache_rows) {
-    if (hq < 1 || hk < 1 || hq % hk || cache_rows < 1) {
+    if (hq < 1 || hk < 1 || hq > 65535 || hq % hk || cache_rows < 1) {
         set_error("%s: bad head counts or cache size (hq=%d hk=%d rows=%d)", who, hq, hk, cache_rows);
         return SCMX_ERR_ARG;
     }

@@ -238,7 +238,7 @@ extern "C" int scmx_attn_prefill(const uint16_t* q, const uint16_t* kcache, cons
         set_error("attn_prefill: null pointer argument");
         return SCMX_ERR_ARG;
     }
-    if (hq < 1 || hk < 1 || hq % hk || d != FA_D) {
+    if (hq < 1 || hk < 1 || hq > 65535 || hq % hk || d != FA_D) {
         set_error("attn_prefill: need hq %% hk == 0 and head dim %d (hq=%d hk=%d d=%d)", FA_D, hq, hk, d);
         return SCMX_ERR_ARG;
     }
@@ -246,8 +246,8 @@ extern "C" int scmx_attn_prefill(const uint16_t* q, const uint16_t* kcache, cons
         set_error("attn_prefill: scale must be positive");
         return SCMX_ERR_ARG;
     }
-    if (L < 0 || off < 0 || off + L > cache_rows) {
-        set_error("attn_prefill: rows %d..%d do not fit a cache of %d rows", off, off + L, cache_rows);
+    if (L < 0 || off < 0 || int64_t(off) + L > cache_rows) {
+        set_error("attn_prefill: rows %d..%lld do not fit a cache of %d rows", off, (long long)off + L, cache_rows);
         return SCMX_ERR_ARG;
     }
     if (uintptr_t(q) % 16 || uintptr_t(kcache) % 16 || uintptr_t(vcache) % 16 || uintptr_t(out) % 8) {

@@ -632,6 +632,7 @@ int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, 
 }
 
 size_t scmx_linear_w4a8_workspace(int M, int K) {
+    if (M <= 0 || K <= 0) return 0;
     const size_t q = (size_t(M) * size_t(K) + 255) & ~size_t(255);
     return q + size_t(M) * sizeof(float);
 }
@@ -720,8 +721,8 @@ static int moe_common(const char* who, const int8_t* xq, const float* xscale, co
         return SCMX_ERR_ARG;
     }
     if (int rc = check_gemm_common(who, R, N, K, epi, true, xq, xscale, wscale, nullptr, out)) return rc;
-    if (!off || !tstart || n_experts < 1 || !(tm == 64 || tm == 128 || tm == 256)) {
-        set_error("%s: need off / tstart, n_experts >= 1 and a row tile of 64, 128 or 256 (got %d)", who, tm);
+    if (!off || !tstart || n_experts < 1 || n_experts > (1 << 20) || !(tm == 64 || tm == 128 || tm == 256)) {
+        set_error("%s: need off / tstart, 1 <= n_experts <= 2^20 and a row tile of 64, 128 or 256 (got %d)", who, tm);
         return SCMX_ERR_ARG;
     }
     *a = GemmArgs{};

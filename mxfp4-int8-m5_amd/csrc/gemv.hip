@@ -742,8 +742,9 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
         set_error("gemv: epilogue %d / prologue %d unknown", epi, pro);
         return SCMX_ERR_ARG;
     }
-    if (N <= 0 || K <= 0 || K % 128 || K % f.block || (K / f.block * f.bc_bits) % 8 || (epi == SCMX_EPI_SWIGLU && N % 4)) {
-        set_error("gemv: need K %% 128 == 0, whole block-code bytes per row, N %% 4 == 0 for SwiGLU (N=%d K=%d)", N, K);
+    if (N <= 0 || N > (1 << 30) || K <= 0 || K > (1 << 20) || K % 128 || K % f.block || (K / f.block * f.bc_bits) % 8 ||
+        (epi == SCMX_EPI_SWIGLU && N % 4)) {
+        set_error("gemv: need N <= 2^30, K <= 2^20, K %% 128 == 0, whole block-code bytes per row, N %% 4 == 0 for SwiGLU (N=%d K=%d)", N, K);
         return SCMX_ERR_ARG;
     }
     if (uintptr_t(codes) % 16 || uintptr_t(x) % 16 || (pro == 2 && uintptr_t(nw) % 16)) {
@@ -752,8 +753,8 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
     }
     int slots = 1;
     if (eidx) {
-        if (batch != 1 || n_eidx < 0 || (xstride != 0 && xstride != 1)) {
-            set_error("gemv: the expert-gather form takes batch 1, xstride 0 or 1");
+        if (batch != 1 || n_eidx < 0 || n_eidx > 65534 || (xstride != 0 && xstride != 1)) {
+            set_error("gemv: the expert-gather form takes batch 1, at most 65534 slots, xstride 0 or 1");
             return SCMX_ERR_ARG;
         }
         slots = n_eidx + (shared_expert >= 0 ? 1 : 0);

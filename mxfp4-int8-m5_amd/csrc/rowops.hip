@@ -589,8 +589,8 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
         set_error("qkv_headnorm: null pointer argument");
         return SCMX_ERR_ARG;
     }
-    if (L < 0 || hq < 1 || hk < 1 || d % 64 || d < 64 || d > 512) {
-        set_error("qkv_headnorm: need head dim a multiple of 64 in 64..512 (d=%d)", d);
+    if (L < 0 || hq < 1 || hk < 1 || hq > 65536 || hk > 65536 || d % 64 || d < 64 || d > 512) {
+        set_error("qkv_headnorm: need 1..65536 heads and a head dim that is a multiple of 64 in 64..512 (hq=%d hk=%d d=%d)", hq, hk, d);
         return SCMX_ERR_ARG;
     }
     if (L == 0) return SCMX_OK;
@@ -607,11 +607,11 @@ int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float*
         set_error("qkv_headnorm_rope: null pointer argument");
         return SCMX_ERR_ARG;
     }
-    if (L < 0 || hq < 1 || hk < 1 || d % 64 || d < 64 || d > 512) {
-        set_error("qkv_headnorm_rope: need head dim a multiple of 64 in 64..512 (d=%d)", d);
+    if (L < 0 || hq < 1 || hk < 1 || hq > 65536 || hk > 65536 || d % 64 || d < 64 || d > 512) {
+        set_error("qkv_headnorm_rope: need 1..65536 heads and a head dim that is a multiple of 64 in 64..512 (hq=%d hk=%d d=%d)", hq, hk, d);
         return SCMX_ERR_ARG;
     }
-    if (cache_rows < L || (!pos_dev && (pos0 < 0 || pos0 + L > cache_rows))) {
+    if (cache_rows < L || (!pos_dev && (pos0 < 0 || pos0 > int64_t(cache_rows) - L))) {
         set_error("qkv_headnorm_rope: rows %lld..%lld do not fit a cache of %d rows", (long long)pos0,
                   (long long)(pos0 + L), cache_rows);
         return SCMX_ERR_ARG;
@@ -628,7 +628,10 @@ int scmx_qkv_fullnorm(const uint16_t* y, const uint16_t* qn, const uint16_t* kn,
         set_error("qkv_fullnorm: null pointer argument");
         return SCMX_ERR_ARG;
     }
-    if (L < 0 || h < 1 || d % 4 || !row_shape_ok("qkv_fullnorm", L, h * d, 16384)) return SCMX_ERR_ARG;
+    if (L < 0 || h < 1 || d < 4 || d % 4 || d > 16384 || h > 16384 / d) {
+        set_error("qkv_fullnorm: need L >= 0, h >= 1, d %% 4 == 0 and h * d <= 16384 (L=%d h=%d d=%d)", L, h, d);
+        return SCMX_ERR_ARG;
+    }
     if (L == 0) return SCMX_OK;
     qkv_fullnorm_kernel<<<dim3(L), dim3(NT), size_t(h) * d * 2 + 72 * 4, (hipStream_t)stream>>>(y, qn, kn, eps, q, k, v, L,
                                                                                                  h, d);
@@ -644,7 +647,7 @@ int scmx_route_topk(const uint16_t* logits, const uint16_t* shared_logit, int M,
         return SCMX_ERR_ARG;
     }
     if (M == 0) return SCMX_OK;
-    route_topk_kernel<<<dim3((M + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, (hipStream_t)stream>>>(
+    route_topk_kernel<<<dim3((unsigned(M) + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, (hipStream_t)stream>>>(
         logits, shared_logit, M, n_experts, topk, renorm, inds, scores);
     return check_launch("route_topk");
 }
@@ -676,10 +679,10 @@ int scmx_route_sort(const int32_t* inds, int M, int topk, int n_experts, int tm,
 int scmx_moe_combine(const uint16_t* y, const int32_t* pos, const uint16_t* scores, const uint16_t* sscore,
                      const uint16_t* res, const uint16_t* w, float eps, uint16_t* h, int8_t* xq, float* xs, int M, int Mp,
                      int K, int topk, void* stream) {
-    if (!y || !pos || !scores || !res || !h || (xq && (!w || !xs)) || Mp < M || topk < 1 ||
+    if (!y || !pos || !scores || !res || !h || (xq && (!w || !xs)) || Mp < M || topk < 1 || topk > 65536 ||
         !row_shape_ok("moe_combine", M, K, 8192)) {
-        if (!(y && pos && scores && res && h) || (xq && (!w || !xs)) || Mp < M || topk < 1)
-            set_error("moe_combine: null pointer argument, Mp < M or topk < 1");
+        if (!(y && pos && scores && res && h) || (xq && (!w || !xs)) || Mp < M || topk < 1 || topk > 65536)
+            set_error("moe_combine: null pointer argument, Mp < M or topk outside 1..65536");
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;

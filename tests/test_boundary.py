@@ -3,8 +3,11 @@ include/scmx.h declares (with the argument counts the ctypes table binds), argum
 before anything is launched, and the host helpers that mirror the reference's call surface (e2e/sc_kernels.py:14-27,
 471-476; e2e/sc_format.py:26-102; e2e/sc_moe.py:155-166) agree with the numpy oracle."""
 import ctypes as C
+import importlib.util
 import os
 import re
+import shutil
+import subprocess
 
 import numpy as np
 import pytest
@@ -130,3 +133,24 @@ def test_attention_split_policy_and_cache_names(pkg):
     assert (f.block, f.bc_bits, tuple(f.mult)) == (16, 4, tuple(range(1, 11)))
     f = PF.sc_format_of("e2m1/B32/pow2")
     assert (f.block, f.bc_bits, tuple(f.mult)) == (32, 2, (1, 2, 4, 8))
+
+
+@pytest.mark.skipif(shutil.which(os.environ.get("HIPCC", "hipcc")) is None, reason="needs hipcc to build the instrumented library")
+def test_host_code_under_address_and_undefined_behaviour_sanitizers():
+    """The library's host code (argument checks, launch-shape arithmetic, dispatch) compiled with AddressSanitizer and
+    UBSan and driven by tests/boundary_driver.cpp on this machine, which has no GPU: every entry point with null
+    pointers, bad shapes and formats, plausible arguments (which end at the failing launch) and 4000 rounds of seeded
+    random integers including the 32-bit extremes.  A sanitizer report aborts the driver; a wrong status makes it
+    exit 1.  Exit 77 = a GPU is present (the driver passes addresses that are not memory), which skips the test."""
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    spec = importlib.util.spec_from_file_location("scmx_build", os.path.join(ROOT, "mxfp4-int8-m5_amd", "build.py"))
+    builder = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(builder)
+    exe = builder.build_host_check(os.path.join(ROOT, "tests", "boundary_driver.cpp"))
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    run = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600, env=env)
+    if run.returncode == 77:
+        pytest.skip("a GPU is present")
+    assert run.returncode == 0, run.stdout[-4000:]
+    assert "0 failure(s)" in run.stdout and "runtime error" not in run.stdout and "AddressSanitizer" not in run.stdout
