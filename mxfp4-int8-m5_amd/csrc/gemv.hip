@@ -16,6 +16,11 @@
 
 namespace scmx {
 
+// Cache policy of the weight loads: the non-temporal hint.  A GEMV reads every code word exactly once, so nothing is
+// gained by keeping the lines; marked as streaming they leave room for the activations and scales that are re-read
+// (lm_head batch 1: 31.0 -> 29.3 us).
+constexpr int W_STREAM = 2;
+
 struct GemvArgs {
     const void* x;            // pro 0: int8 [rows, K]; pro 1, 2: bf16 [rows, K]
     const float* xscale;      // pro 0
@@ -299,7 +304,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
             __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(brow), 0, R * a.bc_row_bytes, 0x00020000);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            it.w[r] = __builtin_amdgcn_raw_buffer_load_b128(rc, int(16u * cc), r * (K / 2), 0);
+            it.w[r] = __builtin_amdgcn_raw_buffer_load_b128(rc, int(16u * cc), r * (K / 2), W_STREAM);
             // the byte with the chunk's block codes: 4 blocks per byte = 4 chunks of 32 weights, or 2 with 16-blocks
             if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> (B16M ? 0 : B16 ? 1 : 2)), r * a.bc_row_bytes, 0);
         }
@@ -561,7 +566,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const GemvArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int c = min(ci * 64 + blk + 16 * i, nchunk - 1);   // past the row: any valid run (its activations are 0)
-            it.w[i] = __builtin_amdgcn_raw_buffer_load_b128(rc, j * (K / 2) + 16 * c, 0, 0);
+            it.w[i] = __builtin_amdgcn_raw_buffer_load_b128(rc, j * (K / 2) + 16 * c, 0, W_STREAM);
         }
         it.bc = __builtin_amdgcn_raw_buffer_load_b128(rb, j * a.bc_row_bytes, ci * 16, 0);   // out of range reads 0
     };
