@@ -53,6 +53,9 @@ def acts(rng, m, k):
     return x
 
 
+WARM_SCALE = 1.0   # --warm-seconds / 0.5: profiler runs set it to 0 so that counter passes see few dispatches
+
+
 def timed(torch, stream, fn, steps, reps=10, warmup=0, warm_s=0.5):
     """fn(i) enqueues one step.  Warm up (`warmup` steps, then until `warm_s` seconds have passed), then time `reps`
     repetitions of `steps` back-to-back steps, each between two events on `stream`.  Returns (median, min) ms per step."""
@@ -62,7 +65,7 @@ def timed(torch, stream, fn, steps, reps=10, warmup=0, warm_s=0.5):
         i += 1
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    while time.perf_counter() - t0 < warm_s:
+    while time.perf_counter() - t0 < warm_s * WARM_SCALE:
         for _ in range(max(1, min(steps, 16))):
             fn(i)
             i += 1
@@ -115,6 +118,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--reps", type=int, default=10, help="timed repetitions of --steps steps (median reported)")
+    ap.add_argument("--warm-seconds", type=float, default=0.5,
+                    help="time-based warm-up of the headline leg (the other legs scale with it); 0 under a profiler")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV leg")
     ap.add_argument("--no-moe", action="store_true", help="skip the grouped mixture-of-experts leg")
@@ -129,6 +134,8 @@ def main():
         print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
         sys.exit(2)
 
+    global WARM_SCALE
+    WARM_SCALE = max(0.0, a.warm_seconds) / 0.5
     import torch
     import mxfp4_int8_m5_amd as pkg
     lib = pkg._lib.load()
