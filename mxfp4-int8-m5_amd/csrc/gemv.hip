@@ -20,6 +20,8 @@ namespace scmx {
 // gained by keeping the lines; marked as streaming they leave room for the activations and scales that are re-read
 // (lm_head batch 1: 31.0 -> 29.3 us).
 constexpr int W_STREAM = 2;
+// From this many weight rows on a layer has enough 16-row groups to keep every CU busy with the half-precision MFMA kernel.
+constexpr int HMFMA_MIN_ROWS = 32768;
 
 struct GemvArgs {
     const void* x;            // pro 0: int8 [rows, K]; pro 1, 2: bf16 [rows, K]
@@ -71,8 +73,12 @@ enum { X_PERM8 = 0, X_HALF = 1, X_PLAIN8 = 2 };
 
 // Stage one activation row into LDS and return its scale: permuted INT8 (8 bytes per 8-group), or with F16 the codes
 // as half-precision values in element order (16 bytes per 8-group).  `red` holds 66 floats.
+// `pre` (valid when have_pre): the thread's 16 bytes of the row, x[8 tid .. 8 tid + 7], loaded by the caller BEFORE it
+// requested its first weights.  Loads return in order, so a row read after the weight prefetch could only be used once
+// those weights had arrived; read first, the row is quantized while the weights are still on their way.
 template <int NT, int XMODE>
-__device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
+__device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red, u32x4 pre = u32x4{0u, 0u, 0u, 0u},
+                           bool have_pre = false) {
     constexpr bool F16 = XMODE == X_HALF;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = a.K;
@@ -124,7 +130,7 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
     }
     // eight values per thread and step, from one 16-byte load (and one of the norm weight for pro 2)
     auto values = [&](int c, float (&v)[8]) {
-        const u32x4 p = *reinterpret_cast<const u32x4*>(xr + 8 * c);
+        const u32x4 p = have_pre ? pre : *reinterpret_cast<const u32x4*>(xr + 8 * c);   // have_pre: only c == tid is asked for
         u32x4 q = u32x4{0u, 0u, 0u, 0u};
         if (a.pro == 2) q = *reinterpret_cast<const u32x4*>(a.nw + 8 * c);
 #pragma unroll
@@ -191,6 +197,143 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red) {
     }
     __syncthreads();   // `red` is reused by the next row
     return s;
+}
+
+// The same staging done by ONE wave (every lane of the wave calls it): with several activation rows each wave of the
+// workgroup takes rows of its own, so the rows are staged side by side instead of one after another and no workgroup
+// barrier is needed in between.  Same arithmetic in the same order as stage_row (maxima are order-free; the sum of
+// squares is formed by the same virtual threads, butterflies and partials), hence the same bits.  K <= 16384.
+// `pre` (valid when have_pre, K <= 512 * WAVE_PRE): the lane's chunks x[8 (lane + 64 j) ..], loaded before the first weights.
+template <int WAVE_PRE>
+struct WavePre {
+    u32x4 v[WAVE_PRE];
+};
+template <int XMODE, int WAVE_PRE>
+__device__ float stage_row_wave(const GemvArgs& a, int row, int8_t* sx, const WavePre<WAVE_PRE>& pre, bool have_pre) {
+    constexpr bool F16 = XMODE == X_HALF;
+    const int lane = threadIdx.x & 63;
+    const int K = a.K;
+    if (a.pro == 0) {
+        const u32x2* src = reinterpret_cast<const u32x2*>(reinterpret_cast<const int8_t*>(a.x) + size_t(row) * K);
+        for (int c = lane; c < K / 8; c += 64) {
+            const u32x2 v = src[c];
+            if (F16) {
+                int q[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = int(int8_t(v[i >> 2] >> (8 * (i & 3))));
+                store_half8(sx + 16 * c, q);
+            } else if (XMODE == X_PLAIN8) {
+                *reinterpret_cast<u32x2*>(sx + 8 * c) = v;
+            } else {
+                *reinterpret_cast<u32x2*>(sx + 8 * c) = u32x2{perm(v[1], v[0], 0x06040200u), perm(v[1], v[0], 0x07050301u)};
+            }
+        }
+        return a.xscale[row];
+    }
+    const uint16_t* xr = reinterpret_cast<const uint16_t*>(a.x) + size_t(row) * K;
+    float inv = 1.0f;
+    if (a.pro == 2) {
+        const int groups = (K / 4 + 63) / 64;
+        float mine = 0.0f;   // lane g keeps the partial of group g
+        for (int g = 0; g < groups; ++g) {
+            const int v = 64 * g + lane;
+            float ss = 0.0f;
+            if (v < K / 4) {
+                const u32x2 p = *reinterpret_cast<const u32x2*>(xr + 4 * v);
+                const float x0 = __uint_as_float(p[0] << 16), x1 = __uint_as_float(p[0] & 0xFFFF0000u);
+                const float x2 = __uint_as_float(p[1] << 16), x3 = __uint_as_float(p[1] & 0xFFFF0000u);
+                ss = __fadd_rn(ss, __fmul_rn(x0, x0));
+                ss = __fadd_rn(ss, __fmul_rn(x1, x1));
+                ss = __fadd_rn(ss, __fmul_rn(x2, x2));
+                ss = __fadd_rn(ss, __fmul_rn(x3, x3));
+            }
+            ss = wave_sum(ss);
+            if (lane == g) mine = ss;
+        }
+        const float tot = wave_sum(lane < groups ? mine : 0.0f);
+        inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(tot, float(K)), a.eps)));
+    }
+    auto values = [&](int c, u32x4 p, float (&v)[8]) {
+        u32x4 q = u32x4{0u, 0u, 0u, 0u};
+        if (a.pro == 2) q = *reinterpret_cast<const u32x4*>(a.nw + 8 * c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float xv = __uint_as_float(i & 1 ? (p[i >> 1] & 0xFFFF0000u) : (p[i >> 1] << 16));
+            if (a.pro == 2) {
+                const float wv = __uint_as_float(i & 1 ? (q[i >> 1] & 0xFFFF0000u) : (q[i >> 1] << 16));
+                v[i] = round_bf16(__fmul_rn(wv, round_bf16(__fmul_rn(xv, inv))));
+            } else {
+                v[i] = xv;
+            }
+        }
+    };
+    const auto emit = [&](int c, const float (&v)[8], float qi) {
+        int q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], qi);
+        if (F16) store_half8(sx + 16 * c, q);
+        else if (XMODE == X_PLAIN8) store_plain8(sx + 8 * c, q);
+        else store_perm8(sx + 8 * c, q);
+    };
+    float amax = 0.0f;
+    if (have_pre) {   // the row is in registers: one pass
+#pragma unroll
+        for (int j = 0; j < WAVE_PRE; ++j)
+            if (lane + 64 * j < K / 8) {
+                float v[8];
+                values(lane + 64 * j, pre.v[j], v);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+            }
+    } else {
+        for (int c = lane; c < K / 8; c += 64) {
+            float v[8];
+            values(c, *reinterpret_cast<const u32x4*>(xr + 8 * c), v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+        }
+    }
+    amax = wave_max(amax);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+    if (have_pre) {
+#pragma unroll
+        for (int j = 0; j < WAVE_PRE; ++j)
+            if (lane + 64 * j < K / 8) {
+                float v[8];
+                values(lane + 64 * j, pre.v[j], v);
+                emit(lane + 64 * j, v, qi);
+            }
+    } else {
+        for (int c = lane; c < K / 8; c += 64) {
+            float v[8];
+            values(c, *reinterpret_cast<const u32x4*>(xr + 8 * c), v);
+            emit(c, v, qi);
+        }
+    }
+    return s;
+}
+
+// The lane's chunks of activation row `row` for stage_row_wave, requested now (prologue 1 only, K <= 512 * WAVE_PRE).
+template <int WAVE_PRE>
+__device__ __forceinline__ bool wave_prefetch_row(const GemvArgs& a, int row, bool valid, WavePre<WAVE_PRE>& pre) {
+    const int lane = threadIdx.x & 63;
+    const bool ok = valid && a.pro == 1 && a.K <= 512 * WAVE_PRE;
+    if (ok) {
+        const uint16_t* xr = reinterpret_cast<const uint16_t*>(a.x) + size_t(row) * a.K;
+#pragma unroll
+        for (int j = 0; j < WAVE_PRE; ++j)
+            if (lane + 64 * j < a.K / 8) pre.v[j] = *reinterpret_cast<const u32x4*>(xr + 8 * (lane + 64 * j));
+    }
+    return ok;
+}
+// The thread's chunk of activation row `row` for the workgroup-wide stage_row (prologue 1 only, K <= 8 * NT).
+template <int NT>
+__device__ __forceinline__ bool block_prefetch_row(const GemvArgs& a, int row, u32x4& pre) {
+    const bool ok = a.pro == 1 && a.K <= 8 * NT;
+    if (ok && int(threadIdx.x) < a.K / 8)
+        pre = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(a.x) + size_t(row) * a.K + 8 * threadIdx.x);
+    return ok;
 }
 
 // Wave sum with DPP adds (one VALU instruction per step): quad swaps, half-row and row mirrors, then the two row
@@ -490,13 +633,16 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         cq[i] = cq[i - 1];
         advance(gq[i], cq[i]);
     }
+    // the first activation row is requested before the weights: memory returns a wave's loads in order
+    u32x4 xpre = u32x4{0u, 0u, 0u, 0u};
+    const bool have_pre = block_prefetch_row<NT>(a, xrow0, xpre);
 #pragma unroll
     for (int i = 0; i < NB; ++i)
         if (gq[i] < groups) load_item(buf[i], gq[i], lane + 64u * cq[i]);
 
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-        const float s = stage_row<NT, FP4 ? X_HALF : X_PERM8>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red);
+        const float s = stage_row<NT, FP4 ? X_HALF : X_PERM8>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red, xpre, have_pre && b == 0);
         for (int c = K * XB / 4 + tid; c < Kp * XB / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp * XB)[c] = 0u;
         if (tid == 0) sxs[b] = s;
     }
@@ -638,15 +784,15 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const GemvArgs a) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
         if (gq[i] < groups) load_item(buf[i], gq[i], cq[i]);
+    const WavePre<1> xpre = {};   // (no early request here: the extra registers would cost this kernel a wave of occupancy)
 
-#pragma unroll
-    for (int b = 0; b < XR; ++b) {
+    for (int b = wave; b < XR; b += NT / 64) {   // a wave per activation row, side by side (rows beyond the batch are zero)
         if (b < BATCH) {
-            const float s = stage_row<NT, X_PLAIN8>(a, b, sx + size_t(b) * Kp, red);
-            for (int c = K / 4 + tid; c < Kp / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
-            if (tid == 0) sxs[b] = s;
+            const float s = stage_row_wave<X_PLAIN8>(a, b, sx + size_t(b) * Kp, xpre, false);
+            for (int c = K / 4 + lane; c < Kp / 4; c += 64) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
+            if (lane == 0) sxs[b] = s;
         } else {
-            for (int c = tid; c < Kp / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
+            for (int c = lane; c < Kp / 4; c += 64) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp)[c] = 0u;
         }
     }
     __syncthreads();
@@ -671,6 +817,210 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const GemvArgs a) {
             cq[i] = cq[1 - i];
             advance(gq[i], cq[i]);
             if (gq[i] < groups) load_item(buf[i], gq[i], cq[i]);
+        }
+    }
+}
+
+// Wide layers in the published format, any batch up to 8: the dot products as half-precision MFMAs.
+// v_cvt_scalef32_pk_f16_fp4 turns a code word into four half-precision pairs, sign and block scale included, which IS the
+// 8-value operand of v_mfma_f32_16x16x32_f16; the activations sit in LDS as half precision (integers up to 127).  Every
+// product is an integer below 2^14 and an accumulator is converted to INT32 and cleared before its sum can reach 2^24
+// (at most 16 MFMAs x 32 products of at most 127 * 96 per chain between two conversions), so the FP32 sums are exact and
+// the totals are the GEMM's INT32 accumulators.  A wave owns 16 consecutive weight rows: lane (row r = l % 16, group
+// c = l / 16) loads 16 bytes of codes (one 32-weight block) per load, load i of a 512-wide piece of K covering
+// k = 128 i + 32 c .. + 31, and feeds each of its four code words to one MFMA whose other operand is the activations of
+// the same 8 k (lane column l % 16 = batch row, columns beyond the batch repeat row 0 and are never stored).  The MFMA
+// sums over the four lane groups, so no cross-lane reduction is left: lane (column b, group c) ends with the totals of
+// batch row b and weight rows 4 c .. 4 c + 3, which is also the unit of the SwiGLU epilogue.
+// Per 8 weights and lane: 4 conversions, one 16-byte LDS read, one MFMA.
+typedef float f4 __attribute__((ext_vector_type(4)));
+// SPLIT (narrow layers): one row group per workgroup, the waves take the 512-wide pieces of K in turn (wave, wave + 4, ...)
+// and their INT32 partial totals meet in LDS: the layer's few rows are spread over 4 x N / 16 waves with one or a few
+// pieces each instead of N / 16 waves walking all of K.
+template <int BATCH, int POL, bool SPLIT, int WAVE_PRE>
+__global__ __launch_bounds__(256) void gemv_hmfma_kernel(const GemvArgs a) {
+    constexpr int NT = 256;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    const int K = a.K, N = a.N;
+    const int Kp = (K + 511) & ~511;                  // whole pieces of 512, zero padded
+    const int pitch = Kp * 2 + 16;                     // bytes per staged row: the 16 spreads the batch rows over the banks
+    int8_t* sx = smem;
+    float* red = reinterpret_cast<float*>(smem + size_t(BATCH) * pitch);   // 68 floats + BATCH scales
+    float* sxs = red + 68;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    // Codes are loaded coalesced (an instruction reads 256 contiguous bytes of each of 4 rows) and turned into the MFMA
+    // layout (lane = row, four lanes per row) through a wave-private LDS slot of 16 rows x 256 bytes; rows are 272 bytes
+    // apart so that the 16 rows a read pass touches fall into different banks.
+    constexpr int WPITCH = 272;
+    int8_t* slot = reinterpret_cast<int8_t*>(sxs + ((BATCH + 3) & ~3)) + size_t(wave) * 16 * WPITCH;
+    const int groups = N / 16;
+    const int CI = Kp / 512;                           // pieces per row group
+    const int g_stride = gridDim.x * (NT / 64);
+    const int brow = r < BATCH ? r : 0;                // the batch row this lane's MFMA column reads
+
+    struct Item {
+        u32x4 w[4];     // loads i = 0..3 of the piece: the 32-weight block 4 i + c of row r
+        uint32_t bc;    // the piece's four block-code bytes of row r (byte i: blocks 4 i .. 4 i + 3)
+    };
+    const auto load_item = [&](Item& it, int g, int ci) {
+        const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + size_t(g) * 16 * (K / 2);   // uniform
+        const uint8_t* brw = a.bcodes + size_t(g) * 16 * a.bc_row_bytes;
+        const __amdgpu_buffer_rsrc_t rc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(crow), 0, 16 * (K / 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rb =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(brw), 0, 16 * a.bc_row_bytes, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)   // rows 4 i .. 4 i + 3: lane l reads 16 bytes at byte 16 (l % 16) of row 4 i + l / 16
+            it.w[i] = __builtin_amdgcn_raw_buffer_load_b128(rc, (4 * i + c) * (K / 2) + 16 * r, ci * 256, POL);
+        it.bc = __builtin_amdgcn_raw_buffer_load_b32(rb, r * a.bc_row_bytes, ci * 4, 0);
+    };
+    f4 acc0, acc1;     // two chains: consecutive MFMAs do not wait for each other
+    int tot[4];
+    const auto flush = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tot[i] += int(acc0[i]) + int(acc1[i]);
+        acc0 = acc1 = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    };
+    const auto compute_item = [&](const Item& it, int ci) {
+        const int8_t* xrow = sx + size_t(brow) * pitch + (size_t(ci) * 512 + 32 * c) * 2;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(slot + (4 * i + c) * WPITCH + 16 * r) = it.w[i];
+        u32x4 wt[4];   // row r, blocks 4 i + c: bytes 64 i + 16 c of the row's 256
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wt[i] = *reinterpret_cast<const u32x4*>(slot + r * WPITCH + 64 * i + 16 * c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float scale = fp4_scale((it.bc >> (8 * i + 2 * c)) & 3u);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t w = wt[i][d];
+                const h2 q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 0);
+                const h2 q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 1);
+                const h2 q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 2);
+                const h2 q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 3);
+                const h8 wv = h8{q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+                const h8 xv = *reinterpret_cast<const h8*>(xrow + (128 * i + 8 * d) * 2);
+                if (d & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xv, acc1, 0, 0, 0);
+                else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xv, acc0, 0, 0, 0);
+            }
+        }
+        flush();   // 8 MFMAs per chain and piece: far below the 43 that keep a chain exact
+    };
+    const auto finish = [&](int g) {
+        if (r >= BATCH) return;
+        const int n = g * 16 + 4 * c;
+        const f4 ws = *reinterpret_cast<const f4*>(a.wscale + n);
+        const float xs = sxs[r];
+        float y[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i] = __fmul_rn(__fmul_rn(float(tot[i]), xs), ws[i]);
+        if (a.epi == SCMX_EPI_SWIGLU) {   // rows (g, g, u, u)
+            const uint16_t o0 = swiglu_bf16(round_bf16(y[0]), round_bf16(y[2]));
+            const uint16_t o1 = swiglu_bf16(round_bf16(y[1]), round_bf16(y[3]));
+            *reinterpret_cast<uint32_t*>(a.out + size_t(r) * (N / 2) + n / 2) = uint32_t(o0) | (uint32_t(o1) << 16);
+            return;
+        }
+        const size_t o = size_t(r) * N + n;
+        if (a.epi == SCMX_EPI_RES) {
+            const u32x2 rr = *reinterpret_cast<const u32x2*>(a.res + o);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float rv = __uint_as_float(i & 1 ? (rr[i >> 1] & 0xFFFF0000u) : (rr[i >> 1] << 16));
+                y[i] = __fadd_rn(rv, round_bf16(y[i]));
+            }
+        }
+        *reinterpret_cast<u32x2*>(a.out + o) = u32x2{uint32_t(f32_to_bf16(y[0])) | (uint32_t(f32_to_bf16(y[1])) << 16),
+                                                      uint32_t(f32_to_bf16(y[2])) | (uint32_t(f32_to_bf16(y[3])) << 16)};
+    };
+
+    const auto advance = [&](int& gi, int& cidx) {
+        if (SPLIT) {
+            cidx += NT / 64;
+            if (cidx >= CI) gi = groups;   // this wave's pieces are done
+        } else if (++cidx == CI) {
+            cidx = 0;
+            gi += g_stride;
+        }
+    };
+    constexpr int NB = 3;   // pieces in flight per wave: 3 x 4 KiB
+    Item buf[NB];
+    int gq[NB], cq[NB];
+    gq[0] = SPLIT ? (wave < CI ? int(blockIdx.x) : groups) : int(blockIdx.x * (NT / 64) + wave);
+    cq[0] = SPLIT ? wave : 0;
+#pragma unroll
+    for (int i = 1; i < NB; ++i) {
+        gq[i] = gq[i - 1];
+        cq[i] = cq[i - 1];
+        advance(gq[i], cq[i]);
+    }
+    // activations are requested before the weights: memory returns a wave's loads in order
+    u32x4 xpre1 = u32x4{0u, 0u, 0u, 0u};
+    constexpr int RPW = BATCH > 4 ? 2 : 1;   // activation rows per wave
+    WavePre<WAVE_PRE> xpre[RPW];
+    bool have_pre = false;
+    if (BATCH == 1) {
+        have_pre = block_prefetch_row<NT>(a, 0, xpre1);
+    } else {
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) have_pre = wave_prefetch_row(a, wave + 4 * j, wave + 4 * j < BATCH, xpre[j]);
+        have_pre = a.pro == 1 && a.K <= 512 * WAVE_PRE;
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+        if (gq[i] < groups) load_item(buf[i], gq[i], cq[i]);
+
+    if (BATCH == 1) {   // one row: the whole workgroup stages it
+        const float s = stage_row<NT, X_HALF>(a, 0, sx, red, xpre1, have_pre);
+        for (int i = K / 2 + tid; i < Kp / 2; i += NT) reinterpret_cast<uint32_t*>(sx)[i] = 0u;
+        if (tid == 0) sxs[0] = s;
+    } else {            // several rows: a wave per row, side by side
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) {
+            const int b = wave + 4 * j;
+            if (b >= BATCH) break;
+            const float s = stage_row_wave<X_HALF>(a, b, sx + size_t(b) * pitch, xpre[j], have_pre);
+            for (int i = K / 2 + lane; i < Kp / 2; i += 64) reinterpret_cast<uint32_t*>(sx + size_t(b) * pitch)[i] = 0u;
+            if (lane == 0) sxs[b] = s;
+        }
+    }
+    __syncthreads();
+    if (!SPLIT && gq[0] >= groups) return;
+    acc0 = acc1 = f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tot[i] = 0;
+    bool more = true;
+    while (more) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            if (gq[i] >= groups) {
+                more = false;
+                break;
+            }
+            compute_item(buf[i], cq[i]);
+            if (!SPLIT && cq[i] == CI - 1) {
+                finish(gq[i]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) tot[v] = 0;
+            }
+            gq[i] = gq[(i + NB - 1) % NB];
+            cq[i] = cq[(i + NB - 1) % NB];
+            advance(gq[i], cq[i]);
+            if (gq[i] < groups) load_item(buf[i], gq[i], cq[i]);
+        }
+    }
+    if constexpr (SPLIT) {   // every wave of the workgroup arrives here: partial totals through the waves' LDS slots
+        *reinterpret_cast<v4i*>(slot + 16 * lane) = v4i{tot[0], tot[1], tot[2], tot[3]};
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int w = 1; w < NT / 64; ++w) {
+                const v4i o = *reinterpret_cast<const v4i*>(slot + size_t(w) * 16 * WPITCH + 16 * lane);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) tot[i] += o[i];
+            }
+            finish(blockIdx.x);
         }
     }
 }
@@ -716,7 +1066,34 @@ static void launch_gemv_mfma(const GemvArgs& a, hipStream_t s) {
 }
 
 template <int BATCH>
+static void launch_gemv_hmfma(const GemvArgs& a, bool split, hipStream_t s) {
+    const int groups = a.N / 16;
+    const int want = (groups + 3) / 4;
+    const int rounds = (want + 1535) / 1536;   // 6 waves per SIMD are resident
+    const dim3 grid(split ? groups : (want + rounds - 1) / rounds), block(256);
+    const size_t smem = size_t(BATCH) * (((a.K + 511) & ~511) * 2 + 16) + (68 + ((BATCH + 3) & ~3)) * sizeof(float) + 4 * 16 * 272;
+    auto go = [&](auto kernel) {
+        if (smem > 64 * 1024)
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
+        kernel<<<grid, block, smem, s>>>(a);
+    };
+    // the early request of the activation rows holds K / 512 chunks per lane: 4 for K <= 2048, 12 up to 6144
+    if (!split) go(gemv_hmfma_kernel<BATCH, W_STREAM, false, 4>);
+    else if (a.K <= 2048) go(gemv_hmfma_kernel<BATCH, W_STREAM, true, 4>);
+    else go(gemv_hmfma_kernel<BATCH, W_STREAM, true, 12>);
+}
+
+template <int BATCH>
 static void launch_gemv_rows(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
+    // wide layers in the published format: half-precision MFMA dot products (whole row groups of 16, pieces of 512)
+    // (several activation rows, K up to 2048: beyond that its half-precision activations cost too much LDS)
+    if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 2048 && a.N >= HMFMA_MIN_ROWS)
+        return launch_gemv_hmfma<BATCH>(a, false, s);
+    // narrow layers with several activation rows: the same kernel with K split over the waves of a workgroup
+    // (batch 1 measured no faster this way than with the per-row kernels: qkv 4.70 against 4.40 us, down 7.32 against 6.34)
+    if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 8192 && a.N < HMFMA_MIN_ROWS &&
+        size_t(BATCH) * a.K <= 32768)
+        return launch_gemv_hmfma<BATCH>(a, true, s);
     if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 4 == 0 && a.K % 512 == 0)
         return launch_gemv_mfma<BATCH>(a, s);
     // more rows per wave = more loads in flight per lane; fewer = more waves for narrow layers
@@ -750,6 +1127,10 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
     if (N <= 0 || N > (1 << 30) || K <= 0 || K > (1 << 20) || K % 128 || K % f.block || (K / f.block * f.bc_bits) % 8 ||
         (epi == SCMX_EPI_SWIGLU && N % 4)) {
         set_error("gemv: need N <= 2^30, K <= 2^20, K %% 128 == 0, whole block-code bytes per row, N %% 4 == 0 for SwiGLU (N=%d K=%d)", N, K);
+        return SCMX_ERR_ARG;
+    }
+    if (pro == 2 && K > 16384) {   // the norm's sum of squares is formed from at most 64 partials of 256 values
+        set_error("gemv: the RMSNorm prologue takes K <= 16384 (K=%d)", K);
         return SCMX_ERR_ARG;
     }
     if (uintptr_t(codes) % 16 || uintptr_t(x) % 16 || (pro == 2 && uintptr_t(nw) % 16)) {

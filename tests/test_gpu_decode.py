@@ -209,3 +209,46 @@ def test_config2_dense_shapes_full_size(G, name, n, k):
     assert np.array_equal(host(G.gemv(dev(xb), dc, db, None, dw, n, 1, pro=1)), ref)
     assert np.array_equal(host(G.gemv(dev(xb)[0], dc, db, None, dw, n, 1, pro=1)), ref[0])
     assert linear.rel_fro(bf16.from_bits(ref[0]), linear.float_reference(bf16.from_bits(xb[:1]), q, ws)[0]) < 1e-2
+
+
+@pytest.mark.parametrize("batch,n,k,pro", [(1, 32768, 512, 0), (1, 40000, 2048, 1), (2, 32784, 1536, 2), (4, 33008, 6144, 1),
+                                           (8, 32768, 1024, 0), (4, 65536, 2048, 2)])
+def test_gemv_wide_layers_every_batch(G, S, batch, n, k, pro):
+    """Layers of 32768 rows and more in the published format run the half-precision-MFMA kernel (16 rows per wave, K in
+    pieces of 512): every output of batch 1 / 2 / 4 / 8 against the oracle with saturated activations, all three
+    prologues, the residual and SwiGLU epilogues, and equal to the narrow-layer kernels on a slice of the same rows."""
+    rng = np.random.default_rng(batch + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    nw = bf16.to_bits(rng.lognormal(0, 0.3, k).astype(F32))
+    if pro == 0:
+        xq = rng.integers(-127, 128, (batch, k)).astype(np.int8)
+        xq[0, :64] = 127
+        xq[-1, -64:] = -127
+        xs = (np.abs(rng.standard_normal(batch)) * 1e-2 + 1e-3).astype(F32)
+        xin, xsc, kw = dev(xq), dev(xs), {}
+    else:
+        xb = bf16.to_bits((rng.standard_normal((batch, k)) * rng.lognormal(0, 1, k)).astype(F32))
+        if pro == 1:
+            xq, xs = linear.act_quant(bf16.from_bits(xb))
+            kw = dict(pro=1)
+        else:
+            xq, xs, _ = linear.rmsnorm_quant(xb, nw, 1e-6, batch)
+            kw = dict(pro=2, nw=dev(nw), eps=1e-6)
+        xin, xsc = dev(xb), None
+    if batch == 1:
+        xin = xin[0]
+    ref1 = linear.gemv(xq, xs, q, ws, 1)
+    y1 = host(G.gemv(xin, dc, db, xsc, dw, n, 1, **kw)).reshape(batch, n)
+    assert np.array_equal(y1, ref1)
+    res = bf16.to_bits(rng.standard_normal((batch, n)).astype(F32))
+    y2 = host(G.gemv(xin, dc, db, xsc, dw, n, 2, res=dev(res if batch > 1 else res[0]), **kw)).reshape(batch, n)
+    assert np.array_equal(y2, linear.gemv(xq, xs, q, ws, 2, res))
+    perm = linear.interleave_gate_up(n // 2)
+    cp = codes.reshape(n, -1)[perm].reshape(-1)
+    y3 = host(G.gemv(xin, dev(cp), dev(bc[perm]), xsc, dev(ws[perm]), n, 3, **kw)).reshape(batch, n // 2)
+    assert np.array_equal(y3, linear.swiglu(ref1[:, :n // 2], ref1[:, n // 2:]))
+    # the first 4096 rows as a narrow layer (the per-row kernels) give the same bits
+    m = 4096
+    ys = host(G.gemv(xin, dev(codes[:m * k // 8]), dev(bc[:m]), xsc, dev(ws[:m]), m, 1, **kw)).reshape(batch, m)
+    assert np.array_equal(ys, y1[:, :m])
