@@ -115,12 +115,16 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // 32-row blocks of this wave's tile that hold rows of the segment (wave-uniform)
     const int mi_active =
         SKIP ? __builtin_amdgcn_readfirstlane(min(MI, max(0, (row_end - (m0 + wm * WTM) + 31) / 32))) : MI;
-    if (a.xscale) {   // published by the barrier that opens the K loop
-        for (int r = tid; r < BM; r += NT) {
-            const int m = m0 + r;
-            s_xs[r] = m < row_end ? a.xscale[a.gather ? a.gather[m] : m] : 0.0f;
-        }
-        for (int c = tid; c < BN; c += NT) s_ws[c] = n0 + c < a.N ? a.wscale[size_t(expert) * a.N + n0 + c] : 0.0f;
+    // The tile's scales are REQUESTED here, before the first operand loads, and stored to LDS after those have been
+    // issued: memory returns a wave's loads in order, so scales requested first arrive first and their wait does not
+    // cover the operand loads (fetched and stored up front they cost every tile two serial round trips to memory).
+    constexpr int XS_PER = (BM + NT - 1) / NT, WS_PER = (BN + NT - 1) / NT;
+    float xs_reg[XS_PER], ws_reg[WS_PER];
+    int xs_row[XS_PER];
+#pragma unroll
+    for (int j = 0; j < XS_PER; ++j) {   // the scale's row: through the gather list when there is one (loaded with the
+        const int m = m0 + tid + j * NT;   // operand rows' entries below, one wait for all of them)
+        xs_row[j] = (a.xscale && tid + j * NT < BM && m < row_end) ? (a.gather ? a.gather[m] : m) : -1;
     }
 
     // ---- per-thread staging assignments (fixed over the K loop) ------------------------------------------------
@@ -170,6 +174,14 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
             b_k[j] = kb * 8 * WPC;
         }
+    }
+
+#pragma unroll
+    for (int j = 0; j < XS_PER; ++j) xs_reg[j] = xs_row[j] >= 0 ? a.xscale[xs_row[j]] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < WS_PER; ++j) {
+        const int c = tid + j * NT;
+        ws_reg[j] = (a.xscale && c < BN && n0 + c < a.N) ? a.wscale[size_t(expert) * a.N + n0 + c] : 0.0f;
     }
 
     // Two register sets hold the global loads of two K steps in flight.
@@ -297,6 +309,14 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // 3 stages x 2 register sets), which keeps every LDS address an immediate offset from a fixed register.
     load_global(r0, 0);
     load_global(r1, BK);
+    if (a.xscale) {   // published by the barrier that opens the K loop
+#pragma unroll
+        for (int j = 0; j < XS_PER; ++j)
+            if (tid + j * NT < BM) s_xs[tid + j * NT] = xs_reg[j];
+#pragma unroll
+        for (int j = 0; j < WS_PER; ++j)
+            if (tid + j * NT < BN) s_ws[tid + j * NT] = ws_reg[j];
+    }
     store_lds(r0, 0, 0);
     store_lds(r1, 1, BK);
     load_global(r0, 2 * BK);
