@@ -252,3 +252,40 @@ def test_gemv_wide_layers_every_batch(G, S, batch, n, k, pro):
     m = 4096
     ys = host(G.gemv(xin, dev(codes[:m * k // 8]), dev(bc[:m]), xsc, dev(ws[:m]), m, 1, **kw)).reshape(batch, m)
     assert np.array_equal(ys, y1[:, :m])
+
+
+@pytest.mark.parametrize("batch,n,k,pro", [(4, 4096, 2048, 0), (2, 2048, 2048, 2), (4, 2048, 6144, 2), (8, 1024, 512, 1),
+                                           (4, 12288, 2048, 1), (2, 48, 1024, 0)])
+def test_gemv_narrow_layers_split_over_k(G, batch, n, k, pro):
+    """Narrow layers with several activation rows (one 16-row group per workgroup, K split over its waves, partial totals
+    through LDS): INT8 input, in-kernel quantization and the RMSNorm prologue, K of one to twelve pieces, every epilogue."""
+    rng = np.random.default_rng(7 * batch + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    nw = bf16.to_bits(rng.lognormal(0, 0.3, k).astype(F32))
+    if pro == 0:
+        xq = rng.integers(-127, 128, (batch, k)).astype(np.int8)
+        xq[0] = 127
+        xs = (np.abs(rng.standard_normal(batch)) * 1e-2 + 1e-3).astype(F32)
+        xin, xsc, kw = dev(xq), dev(xs), {}
+    else:
+        xb = bf16.to_bits((rng.standard_normal((batch, k)) * rng.lognormal(0, 1, k)).astype(F32))
+        xb[-1] = 0                                   # a zero row: scale 0, outputs 0
+        if pro == 1:
+            xq, xs = linear.act_quant(bf16.from_bits(xb))
+            kw = dict(pro=1)
+        else:
+            xq, xs, _ = linear.rmsnorm_quant(xb, nw, 1e-6, batch)
+            kw = dict(pro=2, nw=dev(nw), eps=1e-6)
+        xin, xsc = dev(xb), None
+    ref1 = linear.gemv(xq, xs, q, ws, 1)
+    assert np.array_equal(host(G.gemv(xin, dc, db, xsc, dw, n, 1, **kw)), ref1)
+    res = bf16.to_bits(rng.standard_normal((batch, n)).astype(F32))
+    assert np.array_equal(host(G.gemv(xin, dc, db, xsc, dw, n, 2, res=dev(res), **kw)), linear.gemv(xq, xs, q, ws, 2, res))
+    perm = linear.interleave_gate_up(n // 2)
+    cp = codes.reshape(n, -1)[perm].reshape(-1)
+    y3 = host(G.gemv(xin, dev(cp), dev(bc[perm]), xsc, dev(ws[perm]), n, 3, **kw))
+    assert np.array_equal(y3, linear.swiglu(ref1[:, :n // 2], ref1[:, n // 2:]))
+    for b in range(batch):                           # and every row equals its own batch-1 call
+        one = host(G.gemv(xin[b], dc, db, None if xsc is None else xsc[b:b + 1], dw, n, 1, **kw))
+        assert np.array_equal(one, ref1[b])
