@@ -45,7 +45,10 @@ enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3,
 // SKIP (grouped launches): a row tile that ends inside its expert's segment multiplies only the 32-row blocks that hold
 // valid rows.  The two waves that share a SIMD then own the same columns and different row halves of the tile, so that
 // a half-empty tile halves the MFMA work of every SIMD instead of idling two of the four.
-template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false>
+// PK (B_PACKED_DEFAULT / B_PACKED_B16, K steps of 128): the weights stay packed in LDS -- 64 bytes of codes per row and
+// K step plus the step's block-code bytes -- and every wave decodes its own fragments after reading them.  Half the
+// weight bytes through LDS in both directions, paid with one decode per wave row that shares the fragment.
+template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false>
 __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs a) {
     constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
     constexpr int NT = WGM * WGN * 64;
@@ -61,7 +64,12 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     constexpr int WPC = BN * BK / 32 >= NT ? 4 : 2;
     constexpr int B_CHUNKS = BMODE == B_INT8 ? BN * CPR : BN * BK / (8 * WPC);
     constexpr int B_PER = (B_CHUNKS + NT - 1) / NT;
-    constexpr int STAGE = (BM + BN) * BK;    // bytes per stage: BM activation rows then BN weight rows
+    constexpr int BCB = BMODE == B_PACKED_B16 ? 2 : 1;   // PK: block-code bytes per weight row and K step
+    static_assert(!PK || (BK == 128 && WPC == 4 && (BMODE == B_PACKED_DEFAULT || BMODE == B_PACKED_B16)),
+                  "packed weights in LDS: K steps of 128, 16-byte runs, FP4-conversion formats");
+    // bytes per stage: BM activation rows, then BN weight rows (PK: 64 code bytes each)
+    constexpr int STAGE = BM * BK + (PK ? BN * (BK / 2) : BN * BK);
+    static_assert(STAGE % 16 == 0, "stages keep 16-byte alignment");
 
     // Rows are BK bytes with no padding; the 16-byte chunk c of row r sits at chunk c ^ ((r / RPB) % CPR), which
     // spreads the 16 rows a b128 fragment read touches per pass over all 64 banks.
@@ -74,6 +82,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // round trip to memory
     __shared__ __attribute__((aligned(16))) float s_xs[BM], s_ws[BN];
     auto swz = [](int row, int chunk) { return row * BK + ((chunk ^ ((row / RPB) & (CPR - 1))) << 4); };
+    // packed weight rows (64 bytes, 4 chunks): 4 rows per sweep of the banks, chunk c of row r at c ^ ((r / 4) % 4)
+    auto swzp = [](int row, int chunk) { return row * (BK / 2) + ((chunk ^ ((row >> 2) & 3)) << 4); };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = SKIP ? wave / WGN : wave % WGM, wn = SKIP ? wave % WGN : wave / WGM;
@@ -170,8 +180,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16    ? (kb * 8 * WPC) >> 6
                                              : BMODE == B_PACKED_B16M ? (kb * 8 * WPC) >> 5
                                                                       : 0);
-            b_dst[j] = BM * BK + swz(row, kb * WPC / 2);
-            b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
+            if (PK) {   // the run's 16 code bytes as they are
+                b_dst[j] = BM * BK + swzp(row, kb);
+                b_dst2[j] = 0;
+            } else {
+                b_dst[j] = BM * BK + swz(row, kb * WPC / 2);
+                b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
+            }
             b_k[j] = kb * 8 * WPC;
         }
     }
@@ -215,6 +230,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                         r.b[j][0] = v[0];
                         r.b[j][1] = v[1];
                     }
+                    if (PK) continue;   // block codes go straight to the lanes that decode
                     if (BMODE == B_PACKED_DEFAULT)   // 32-blocks, 2-bit codes, 4 blocks per byte: keep the raw byte
                         r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 7, 0);
                     if (BMODE == B_PACKED_B16)       // 16-blocks: a byte covers 64 weights
@@ -245,6 +261,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             if (B_CHUNKS % NT == 0 || tid + j * NT < B_CHUNKS) {
                 if (BMODE == B_INT8) {
                     if (q == 0) *reinterpret_cast<u32x4*>(st + b_dst[j]) = r.b[j];
+                } else if (PK) {
+                    if (q == j % NKK) *reinterpret_cast<u32x4*>(st + b_dst[j]) = r.b[j];
                 } else {
 #pragma unroll
                     for (int w = 0; w < WPC; ++w) {
@@ -307,6 +325,19 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // after it was written, so the first fragments of step kt+1 are fetched at the end of iteration kt, ahead of the
     // barrier that opens kt+1.  The stage indices are compile-time constants (the loop is unrolled over the
     // 3 stages x 2 register sets), which keeps every LDS address an immediate offset from a fixed register.
+    [[maybe_unused]] uint32_t bcc[NI], bcn[NI];   // PK: block codes of the current / the next two K steps
+    [[maybe_unused]] int bc_src[NI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) bc_src[j] = min(n0 + wn * WTN + j * 32 + lr, a.N - 1) * a.bc_row_bytes;
+    // block codes of K steps s and s + 1 (s even); past the end the last pair of steps again (never consumed)
+    auto load_bc = [&](int s, uint32_t (&f)[NI]) {
+        const int so = min(s, (K / BK - 1) & ~1) * BCB;
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            f[j] = BCB == 2 ? uint32_t(__builtin_amdgcn_raw_buffer_load_b32(rbc, bc_src[j], so, 0))
+                            : uint32_t(__builtin_amdgcn_raw_buffer_load_b16(rbc, bc_src[j], so, 0));
+    };
+    if constexpr (PK) load_bc(0, bcc);   // ahead of the operand loads, like the scales
     load_global(r0, 0);
     load_global(r1, BK);
     if (a.xscale) {   // published by the barrier that opens the K loop
@@ -321,11 +352,110 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     store_lds(r1, 1, BK);
     load_global(r0, 2 * BK);
     load_global(r1, 3 * BK);
+    // ---- PK: fragments of packed weights ------------------------------------------------------------------------
+    // The k positions of a 64-wide pair of MFMA slices are dealt so that a lane's packed codes are one 16-byte read:
+    // lane half h supplies k = 64 kp + 32 h + 16 s + (0..15) to slice s of pair kp, i.e. 32 consecutive activation
+    // bytes (two 16-byte reads) and 32 consecutive codes (one), the latter one 32-block or two 16-blocks.
+    constexpr int NKP = NKK / 2;
+    // Three things are in flight per wave: the MFMAs of pair p, the decode of pair p + 1 (its codes were read during
+    // pair p - 1) and the LDS reads of pair p + 1's activations and pair p + 2's codes.
+    // The block codes do not pass through LDS: the lane that decodes row n reads the codes of two K steps of that row
+    // (2 * BCB bytes) from memory every second step, two steps ahead.
+    [[maybe_unused]] v4i pa[2][2][MI];   // activation fragments [pair parity][slice][32-row block]
+    [[maybe_unused]] v4i pw[2][NI];      // 32 codes per weight row as read from LDS [pair parity]
+    [[maybe_unused]] v4i px[2][2][NI];   // decoded INT8 operands [pair parity][slice][32-column block]
+    [[maybe_unused]] int koff_pa[NKP][2], koff_pw[NKP];
+#pragma unroll
+    for (int kp = 0; kp < NKP; ++kp) {
+        koff_pa[kp][0] = ((4 * kp + 2 * half) ^ sw) << 4;
+        koff_pa[kp][1] = ((4 * kp + 2 * half + 1) ^ sw) << 4;
+        koff_pw[kp] = ((2 * kp + half) ^ ((lr >> 2) & 3)) << 4;
+    }
+    [[maybe_unused]] const int w_frag = BM * BK + (wn * WTN + lr) * (BK / 2);
+    auto load_pa = [&](const int8_t* src, int kp, v4i (&f)[2][MI]) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+            if (!SKIP || i < mi_active) {
+                f[0][i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff_pa[kp][0]);
+                f[1][i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff_pa[kp][1]);
+            }
+    };
+    auto load_pw = [&](const int8_t* src, int kp, v4i (&f)[NI]) {
+        if (SKIP && mi_active == 0) return;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) f[j] = *reinterpret_cast<const v4i*>(src + w_frag + j * 32 * (BK / 2) + koff_pw[kp]);
+    };
+    // 32 codes -> the INT8 operands of the pair's two slices; `odd` = the K step's parity (which half of the block codes)
+    auto decode_pair = [&](const v4i (&f)[NI], const uint32_t (&bc)[NI], int odd, int kp, v4i (&x)[2][NI]) {
+        if (SKIP && mi_active == 0) return;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            float s0, s1;
+            if (BMODE == B_PACKED_B16) {   // blocks 4 kp + 2 h and the next one of the step's 8
+                const uint32_t t = bc[j] >> (16 * odd + 8 * kp + 4 * half);
+                s0 = fp4_scale(t & 3u);
+                s1 = fp4_scale((t >> 2) & 3u);
+            } else {                       // block 2 kp + h of the step's 4
+                s0 = s1 = fp4_scale((bc[j] >> (8 * odd + 4 * kp + 2 * half)) & 3u);
+            }
+            uint32_t o[8];
+            decode_word_fp4(uint32_t(f[j][0]), s0, o[0], o[1]);
+            decode_word_fp4(uint32_t(f[j][1]), s0, o[2], o[3]);
+            decode_word_fp4(uint32_t(f[j][2]), s1, o[4], o[5]);
+            decode_word_fp4(uint32_t(f[j][3]), s1, o[6], o[7]);
+            x[0][j] = v4i{int(o[0]), int(o[1]), int(o[2]), int(o[3])};
+            x[1][j] = v4i{int(o[4]), int(o[5]), int(o[6]), int(o[7])};
+        }
+    };
+    auto iteration_pk = [&](auto step_tag, auto parity_tag, Staged& r, int kt) {
+        constexpr int rd = decltype(step_tag)::value;
+        constexpr int odd = decltype(parity_tag)::value;   // kt % 2
+        constexpr int wr = (rd + 2) % NSTAGE;
+        constexpr int nx = (rd + 1) % NSTAGE;
+        __syncthreads();
+        const int8_t* src = smem + rd * STAGE;
+        const int8_t* nxt = smem + nx * STAGE;
+        int8_t* dst = smem + wr * STAGE;
+        const int k2 = min((kt + 2) * BK, K - BK);
+        const int k4 = min((kt + 4) * BK, K - BK);
+        uint32_t o[B_PER][8];
+        if (!odd) load_bc(kt + 2, bcn);
+#pragma unroll
+        for (int kp = 0; kp < NKP; ++kp) {
+            const int cur = kp % 2, oth = (kp + 1) % 2;   // NKP is even: pair 0 of every step has parity 0
+            if (kp + 1 < NKP) {
+                load_pa(src, kp + 1, pa[oth]);
+                decode_pair(pw[oth], bcc, odd, kp + 1, px[oth]);
+            } else {   // pair 0 of step kt + 1
+                load_pa(nxt, 0, pa[oth]);
+                if (odd) {
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) bcc[j] = bcn[j];
+                }
+                decode_pair(pw[oth], bcc, 1 - odd, 0, px[oth]);
+            }
+            load_pw(nxt, kp, pw[cur]);   // pair kp + 2 = pair kp of the next step; pw[cur] was decoded a pair ago
+#pragma unroll
+            for (int sl = 0; sl < 2; ++sl) {
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    if (SKIP && i >= mi_active) continue;
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(px[cur][sl][j], pa[cur][sl][i], acc[i][j], 0, 0, 0);
+                }
+                stage_slice(r, dst, k2, 2 * kp + sl, o);
+            }
+        }
+        load_global(r, k4);
+    };
+    static_assert(!PK || NKP % 2 == 0, "the pair buffers return to phase 0 every K step");
+
     // Fragments are fetched FD - 1 k slices ahead of the MFMAs that use them, into FD rotating register buffers; the
     // slices fetched at the end of an iteration belong to the next step's stage.
     constexpr int AHEAD = FD - 1;
     static_assert(AHEAD >= 1 && AHEAD <= NKK, "fragment prefetch distance");
-    v4i fa[FD][MI], fb[FD][NI];
+    [[maybe_unused]] v4i fa[FD][MI], fb[FD][NI];
     auto load_frags = [&](const int8_t* src, int kk, v4i (&xa)[MI], v4i (&xb)[NI]) {
         if (SKIP && mi_active == 0) return;
 #pragma unroll
@@ -335,9 +465,16 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         for (int j = 0; j < NI; ++j) xb[j] = *reinterpret_cast<const v4i*>(src + b_frag + j * 32 * BK + koff[kk]);
     };
     __syncthreads();
+    if constexpr (PK) {
+        load_pa(smem, 0, pa[0]);
+        load_pw(smem, 0, pw[0]);
+        load_pw(smem, 1, pw[1]);
+        decode_pair(pw[0], bcc, 0, 0, px[0]);
+    } else {
 #pragma unroll
-    for (int q = 0; q < AHEAD; ++q) load_frags(smem, q, fa[q], fb[q]);
-    auto iteration = [&](auto step_tag, Staged& r, int kt) {
+        for (int q = 0; q < AHEAD; ++q) load_frags(smem, q, fa[q], fb[q]);
+    }
+    auto iteration_staged = [&](auto step_tag, Staged& r, int kt) {
         constexpr int rd = decltype(step_tag)::value;        // kt % 3: stage of step kt
         constexpr int wr = (rd + 2) % NSTAGE;                // stage of step kt + 2
         constexpr int nx = (rd + 1) % NSTAGE;                // stage of step kt + 1
@@ -368,6 +505,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         }
         load_global(r, k4);
     };
+    auto iteration = [&](auto step_tag, auto parity_tag, Staged& r, int kt) {
+        if constexpr (PK) iteration_pk(step_tag, parity_tag, r, kt); else iteration_staged(step_tag, r, kt);
+    };
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     using S2 = std::integral_constant<int, 2>;
@@ -375,23 +515,25 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // iteration has exactly one predecessor.  (With merging paths the compiler must assume the fewest outstanding
     // loads of any path when it places its waits, and ends up waiting for loads issued one step ago.)
     int kt = 0;
-    for (; kt + 6 <= KT; kt += 6) {
-        iteration(S0{}, r0, kt);
-        iteration(S1{}, r1, kt + 1);
-        iteration(S2{}, r0, kt + 2);
-        iteration(S0{}, r1, kt + 3);
-        iteration(S1{}, r0, kt + 4);
-        iteration(S2{}, r1, kt + 5);
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
+    for (; kt + 6 <= KT; kt += 6) {   // kt stays even here: the parity of every copy is fixed
+        iteration(S0{}, Even{}, r0, kt);
+        iteration(S1{}, Odd{}, r1, kt + 1);
+        iteration(S2{}, Even{}, r0, kt + 2);
+        iteration(S0{}, Odd{}, r1, kt + 3);
+        iteration(S1{}, Even{}, r0, kt + 4);
+        iteration(S2{}, Odd{}, r1, kt + 5);
     }
     if (kt < KT) {
-        iteration(S0{}, r0, kt);
+        iteration(S0{}, Even{}, r0, kt);
         if (kt + 1 < KT) {
-            iteration(S1{}, r1, kt + 1);
+            iteration(S1{}, Odd{}, r1, kt + 1);
             if (kt + 2 < KT) {
-                iteration(S2{}, r0, kt + 2);
+                iteration(S2{}, Even{}, r0, kt + 2);
                 if (kt + 3 < KT) {
-                    iteration(S0{}, r1, kt + 3);
-                    if (kt + 4 < KT) iteration(S1{}, r0, kt + 4);
+                    iteration(S0{}, Odd{}, r1, kt + 3);
+                    if (kt + 4 < KT) iteration(S1{}, Even{}, r0, kt + 4);
                 }
             }
         }
@@ -530,23 +672,30 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
 
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false>
+template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false>
 static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStream_t s) {
     GemmArgs a = a_in;
     if (a.epi == SCMX_EPI_SWIGLU) a.silu = silu_table_device();
     const int num_n = (a.N + BN - 1) / BN;
     if (a.tstart) row_tiles = (row_tiles + 7) & ~7;   // grouped: whole chunks of 8 row-tile slots (spare slots exit at once)
     const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * 64);
-    if (bmode == B_INT8)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
-    else if (bmode == B_PACKED_DEFAULT)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
-    else if (bmode == B_PACKED_B16)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
-    else if (bmode == B_PACKED_B16M)
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
-    else
-        gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+    if constexpr (PK) {   // callers choose this tile for the two FP4-conversion formats only
+        if (bmode == B_PACKED_DEFAULT)
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
+        else
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
+    } else {
+        if (bmode == B_INT8)
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+        else if (bmode == B_PACKED_DEFAULT)
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+        else if (bmode == B_PACKED_B16)
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+        else if (bmode == B_PACKED_B16M)
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+        else
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+    }
 }
 
 static int packed_mode(const DevFormat& f) {
@@ -759,6 +908,11 @@ static void launch_grouped(const GemmArgs& a, int bmode, int tm, hipStream_t s) 
         launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
     else if (tm == 128)
         launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
+    else if ((bmode == B_PACKED_DEFAULT || bmode == B_PACKED_B16) && a.K % 256 == 0 && a.N % 256 == 0)
+        // few rows per expert: the pass streams the expert weights, and what it pays per weight is the staging.  The
+        // packed tile writes and reads half the weight bytes in LDS, its eight waves sit side by side along N (every
+        // fragment is decoded once) and two workgroups share a CU (128 registers).
+        launch_tile<64, 256, 128, 1, 8, 4, 2, false, true>(a, bmode, max_tiles, s);
     else
         launch_tile<64, 128, 128, 2, 4>(a, bmode, max_tiles, s);
 }

@@ -350,3 +350,37 @@ def test_grouped_gemm_random_segments(M):
         got = host(M.moe_mm(dev(xq), r, dev(codes), dev(bc), dev(ws), off, tstart, mt, n, epi, dev(xs), tile=(tm, 64, 4)))
         want = ref if epi == 0 else moe.moe_epilogue(ref, xs, ws, ex, epi)
         assert np.array_equal(got, want), (case, e, n, k, tm, epi, counts.tolist())
+
+
+@pytest.mark.parametrize("fi", [0, 1])
+def test_packed_weight_tile_of_64_row_passes(M, fi):
+    """Row tile 64 with the published codebook (32- and 16-element blocks), N % 256 == 0 and K % 256 == 0 takes the
+    kernel that keeps the weights packed in LDS and decodes them per wave after the fragment read, with the block
+    codes read by the decoding lanes two K steps at a time.  Segments of 0 / 1 / 31 / 33 / 64 / 65 / 130 / 200 rows,
+    every number of K steps from 2 to 14 that the loop structure distinguishes (whole trips of 6 and each tail), a
+    gather list, INT32 / scaled / SwiGLU epilogues: bit-exact against the oracle (e2e/sc_moe.py:19-92)."""
+    fmt = FORMATS[fi]
+    rng = np.random.default_rng(640 + fi)
+    counts = np.array([33, 0, 1, 64, 31, 200, 65, 0, 130])
+    e = len(counts)
+    ex = np.repeat(np.arange(e), counts).astype(np.int32)
+    r = len(ex)
+    off, tstart, mt = M.segments(dev(ex), e, 64)
+    for n, k in [(256, 256), (512, 512), (256, 768), (256, 1024), (512, 1280), (256, 1536), (256, 1792), (768, 2048)]:
+        packs = [random_packed(rng, n, k, fmt) for _ in range(e)]
+        codes, bc, ws = (np.stack([p[i] for p in packs]) for i in range(3))
+        wq = np.stack([p[3] for p in packs])
+        src = rng.integers(-127, 128, (r + 40, k)).astype(np.int8)     # the rows are gathered out of a larger matrix
+        tok = rng.permutation(r + 40)[:r].astype(np.int32)
+        ss = (np.abs(rng.standard_normal(r + 40)) * 1e-2).astype(F32)
+        xq, xs = src[tok], ss[tok]
+        ref = moe.moe_int_gemm(xq, ex, wq)
+        dc, db, dw, pf = dev(codes), dev(bc), dev(ws), product_format(fmt)
+        acc = host(M.moe_mm(dev(src), r, dc, db, dw, off, tstart, mt, n, 0, tile=(64, 64, 4), gather=dev(tok), fmt=pf))
+        assert np.array_equal(acc, ref), (n, k)
+        for epi in (1, 3):
+            y = host(M.moe_mm(dev(src), r, dc, db, dw, off, tstart, mt, n, epi, dev(ss), tile=(64, 64, 4), gather=dev(tok), fmt=pf))
+            assert np.array_equal(y, moe.moe_epilogue(ref, xs, ws, ex, epi)), (n, k, epi)
+        # without the gather list, rows in place
+        acc = host(M.moe_mm(dev(xq), r, dc, db, dw, off, tstart, mt, n, 0, tile=(64, 64, 4), fmt=pf))
+        assert np.array_equal(acc, ref), (n, k, "in place")
