@@ -908,10 +908,12 @@ static void launch_grouped(const GemmArgs& a, int bmode, int tm, hipStream_t s) 
         launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
     else if (tm == 128)
         launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, max_tiles, s);
-    else if ((bmode == B_PACKED_DEFAULT || bmode == B_PACKED_B16) && a.K % 256 == 0 && a.N % 256 == 0)
+    else if ((bmode == B_PACKED_DEFAULT || bmode == B_PACKED_B16) && a.K % 256 == 0 && a.N % 256 == 0 &&
+             reinterpret_cast<uintptr_t>(a.bcodes) % 4 == 0)
         // few rows per expert: the pass streams the expert weights, and what it pays per weight is the staging.  The
         // packed tile writes and reads half the weight bytes in LDS, its eight waves sit side by side along N (every
-        // fragment is decoded once) and two workgroups share a CU (128 registers).
+        // fragment is decoded once) and two workgroups share a CU (128 registers).  Its lanes read the block codes of two
+        // K steps with one aligned 2- or 4-byte load, hence the conditions on K and on the pointer.
         launch_tile<64, 256, 128, 1, 8, 4, 2, false, true>(a, bmode, max_tiles, s);
     else
         launch_tile<64, 128, 128, 2, 4>(a, bmode, max_tiles, s);

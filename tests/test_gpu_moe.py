@@ -384,3 +384,8 @@ def test_packed_weight_tile_of_64_row_passes(M, fi):
         # without the gather list, rows in place
         acc = host(M.moe_mm(dev(xq), r, dc, db, dw, off, tstart, mt, n, 0, tile=(64, 64, 4), fmt=pf))
         assert np.array_equal(acc, ref), (n, k, "in place")
+        # block codes at an odd address: the aligned two-step reads of that kernel are not possible, the result is the same
+        odd = torch.empty(db.numel() + 1, dtype=torch.uint8, device="cuda")[1:].view(db.shape)
+        odd.copy_(db)
+        acc = host(M.moe_mm(dev(xq), r, dc, odd, dw, off, tstart, mt, n, 0, tile=(64, 64, 4), fmt=pf))
+        assert np.array_equal(acc, ref), (n, k, "odd block-code address")
