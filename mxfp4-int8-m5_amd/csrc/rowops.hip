@@ -429,14 +429,27 @@ __global__ __launch_bounds__(NT) void moe_combine_kernel(const uint16_t* __restr
         u32x2 o = r2;
         if (row < M) {
             float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (int j = 0; j < topk; ++j) {
-                const int p = pos[row * topk + j];
-                const float sc = bf16_to_f32((sscore && j == topk - 1) ? sscore[row] : scores[row * nsc + j]);
-                const u32x2 y2 = *reinterpret_cast<const u32x2*>(y + size_t(p) * K + 4 * c);
+            // the slots' rows are requested eight at a time, then added in slot order
+            for (int j0 = 0; j0 < topk; j0 += 8) {
+                u32x2 y2[8];
+                float sc[8];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float yv = __uint_as_float(i & 1 ? (y2[i >> 1] & 0xFFFF0000u) : (y2[i >> 1] << 16));
-                    acc[i] = round_bf16(__fadd_rn(round_bf16(__fmul_rn(yv, sc)), acc[i]));
+                for (int u = 0; u < 8; ++u) {
+                    const int j = j0 + u;
+                    if (j < topk) {
+                        const int p = pos[row * topk + j];
+                        sc[u] = bf16_to_f32((sscore && j == topk - 1) ? sscore[row] : scores[row * nsc + j]);
+                        y2[u] = *reinterpret_cast<const u32x2*>(y + size_t(p) * K + 4 * c);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (j0 + u >= topk) break;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float yv = __uint_as_float(i & 1 ? (y2[u][i >> 1] & 0xFFFF0000u) : (y2[u][i >> 1] << 16));
+                        acc[i] = round_bf16(__fadd_rn(round_bf16(__fmul_rn(yv, sc[u])), acc[i]));
+                    }
                 }
             }
             uint16_t hb[4];
