@@ -240,8 +240,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                 }
             }
     };
-    // Loads past the last K step re-read the last step (never consumed): every iteration issues the same loads, so
-    // the wait before a register set is used covers exactly that set and not the younger one.
     auto load_global = [&](Staged& r, int k0) {
         k0 = min(k0, K - BK);
 #pragma unroll
