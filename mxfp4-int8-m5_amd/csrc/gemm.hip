@@ -149,11 +149,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                                                       : rsrc(reinterpret_cast<const uint8_t*>(a.codes) + erow * (K / 2), size_t(a.N) * (K / 2));
     const __amdgpu_buffer_rsrc_t rbc = rsrc(a.bcodes + erow * a.bc_row_bytes, size_t(a.N) * a.bc_row_bytes);
     int a_src[A_PER], a_dst[A_PER];
+    uint32_t a_live = 0;   // SKIP: the chunks of rows inside the segment (the others are neither written to LDS nor used)
 #pragma unroll
     for (int j = 0; j < A_PER; ++j) {
         const int c = tid + j * NT;
         const int row = c / CPR, kc = c % CPR;
-        int gr = min(m0 + row, a.M - 1);
+        if (m0 + row < row_end) a_live |= 1u << j;
+        int gr = min(m0 + row, row_end - 1);   // rows past the segment re-read its last row: one cache line, not a row each
         if (a.gather) gr = a.gather[gr];
         a_src[j] = int(uint32_t(gr) * uint32_t(K) + kc * 16);
         a_dst[j] = swz(row, kc);
@@ -252,7 +254,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     auto stage_slice = [&](const Staged& r, int8_t* st, int k0, int q, uint32_t (&o)[B_PER][8]) {
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
-            if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS))
+            if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS) && (!SKIP || ((a_live >> j) & 1u)))
                 *reinterpret_cast<u32x4*>(st + a_dst[j]) = r.a[j];
 #pragma unroll
         for (int j = 0; j < B_PER; ++j)
