@@ -4,6 +4,8 @@
 // Reduction order (fixed, so results do not depend on the launch shape): a row's sum of squares is formed by K/4
 // virtual threads of 4 consecutive values summed in order, 64 virtual threads per butterfly wave sum, and one more
 // butterfly over the per-group partials.
+#include <type_traits>
+
 #include "scmx_common.h"
 
 namespace scmx {
@@ -484,11 +486,14 @@ static bool row_shape_ok(const char* who, int rows, int K, int max_k) {
 // taken per lane in rising j and then by the butterfly wave_sum.  The k winners are found by k wave-wide maxima over
 // the key (probability bits << 16 | 65535 - j): largest probability first, equal ones by rising expert index.
 constexpr int ROUTE_MAX_E = 1024;
+// PER = experts per lane the kernel is built for (64 * PER >= E): slots past E cost what live ones do, so the launch picks
+// the smallest of 1, 2, 4, 8, 16 that covers E.  The arithmetic of the live slots does not depend on PER.
+template <int PER>
 __global__ __launch_bounds__(NT) void route_topk_kernel(const uint16_t* __restrict__ logits,
                                                         const uint16_t* __restrict__ shared_logit, int M, int E, int topk,
                                                         int renorm, int32_t* __restrict__ inds,
                                                         uint16_t* __restrict__ scores) {
-    constexpr int PER = ROUTE_MAX_E / 64;
+    static_assert(PER >= 1 && 64 * PER <= ROUTE_MAX_E, "experts per lane");
     const int lane = threadIdx.x & 63, t = blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
     if (t >= M) return;   // wave-uniform
     const int stride = topk + (shared_logit ? 1 : 0);
@@ -660,8 +665,17 @@ int scmx_route_topk(const uint16_t* logits, const uint16_t* shared_logit, int M,
         return SCMX_ERR_ARG;
     }
     if (M == 0) return SCMX_OK;
-    route_topk_kernel<<<dim3((unsigned(M) + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, (hipStream_t)stream>>>(
-        logits, shared_logit, M, n_experts, topk, renorm, inds, scores);
+    const dim3 grid((unsigned(M) + NT / 64 - 1) / (NT / 64)), block(NT);
+    hipStream_t st = (hipStream_t)stream;
+    const auto launch = [&](auto per_tag) {
+        route_topk_kernel<decltype(per_tag)::value><<<grid, block, 0, st>>>(logits, shared_logit, M, n_experts, topk, renorm,
+                                                                           inds, scores);
+    };
+    if (n_experts <= 64) launch(std::integral_constant<int, 1>{});
+    else if (n_experts <= 128) launch(std::integral_constant<int, 2>{});
+    else if (n_experts <= 256) launch(std::integral_constant<int, 4>{});
+    else if (n_experts <= 512) launch(std::integral_constant<int, 8>{});
+    else launch(std::integral_constant<int, 16>{});
     return check_launch("route_topk");
 }
 
