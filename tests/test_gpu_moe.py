@@ -47,7 +47,10 @@ def test_route_sort_contract(M, m, topk, e, tm):
 
 @pytest.mark.parametrize("m,e,k,renorm,shared", [(4096, 64, 8, True, False), (2048, 256, 8, True, True), (4096, 64, 8, False, False),
                                                  (1, 64, 8, True, False), (77, 257, 9, True, False), (300, 1000, 64, False, True), (40, 1024, 3, True, False),
-                                                 (129, 8, 8, True, True), (50, 5, 1, True, False)])
+                                                 (129, 8, 8, True, True), (50, 5, 1, True, False),
+                                                 # the sizes either side of each build of the kernel (1, 2, 4, 8, 16 experts per lane)
+                                                 (33, 65, 4, True, False), (20, 128, 8, True, True), (10, 129, 2, False, False),
+                                                 (12, 512, 8, True, False), (9, 513, 6, True, True)])
 def test_router_against_oracle(M, m, e, k, renorm, shared):
     """Softmax -> top-k -> renormalisation (-> shared-expert slot with its sigmoid gate) on config 3 / config 4 router
     logits (N(0,1) + N(0,1.5) expert bias, bf16): expert indices and bf16 scores bit for bit against the oracle
