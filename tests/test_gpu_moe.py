@@ -392,3 +392,37 @@ def test_packed_weight_tile_of_64_row_passes(M, fi):
         odd.copy_(db)
         acc = host(M.moe_mm(dev(xq), r, dc, odd, dw, off, tstart, mt, n, 0, tile=(64, 64, 4), fmt=pf))
         assert np.array_equal(acc, ref), (n, k, "odd block-code address")
+
+
+def test_packed_weight_tile_random_layouts(M):
+    """Sixteen seeded random expert layouts at row tile 64 on shapes that take the packed-weight kernel and on neighbours
+    that do not (N or K not a multiple of 256): both block sizes, 1 to 23 experts, segments of 0 to 300 rows, gather list
+    or rows in place, EPI 0 / 1 / 3: bit-exact against the oracle."""
+    rng = np.random.default_rng(6464)
+    for case in range(16):
+        fmt = FORMATS[int(rng.integers(0, 2))]
+        e = int(rng.integers(1, 24))
+        n = int(rng.choice([256, 512, 768, 1024, 384, 128]))
+        k = int(rng.choice([256, 512, 768, 1280, 2048, 2304, 384, 640]))
+        counts = rng.integers(0, 150, e)
+        counts[rng.integers(0, e)] = int(rng.choice([0, 1, 64, 65, 300]))
+        if counts.sum() == 0:
+            counts[0] = 3
+        ex = np.repeat(np.arange(e), counts).astype(np.int32)
+        r = len(ex)
+        packs = [random_packed(rng, n, k, fmt) for _ in range(e)]
+        codes, bc, ws = (np.stack([p[i] for p in packs]) for i in range(3))
+        wq = np.stack([p[3] for p in packs])
+        extra = int(rng.integers(0, 50))
+        src = rng.integers(-127, 128, (r + extra, k)).astype(np.int8)
+        tok = rng.permutation(r + extra)[:r].astype(np.int32)
+        ss = (np.abs(rng.standard_normal(r + extra)) * 1e-2).astype(F32)
+        gathered = bool(rng.integers(0, 2))
+        xq, xs = (src[tok], ss[tok]) if gathered else (src[:r], ss[:r])
+        off, tstart, mt = M.segments(dev(ex), e, 64)
+        epi = int(rng.choice([0, 1, 3]))
+        ref = moe.moe_int_gemm(xq, ex, wq)
+        want = ref if epi == 0 else moe.moe_epilogue(ref, xs, ws, ex, epi)
+        got = host(M.moe_mm(dev(src), r, dev(codes), dev(bc), dev(ws), off, tstart, mt, n, epi, dev(ss), tile=(64, 64, 4),
+                            gather=dev(tok) if gathered else None, fmt=product_format(fmt)))
+        assert np.array_equal(got, want), (case, fmt.block, e, n, k, epi, gathered, counts.tolist())
