@@ -16,12 +16,21 @@ Module map (reference files are cited as path:line inside each function):
 Parity status
   pinned by golden vectors written from the reference's own numpy modules (tests/golden/):
       quantizer.*  layout.*  family.quantize  family.pack_parts  linear.act_quant (via reference quant_ref formula)
-  pinned by closed forms / brute force (tests/test_oracle_*.py):
+  pinned by closed forms / brute force / an independent bf16 implementation (tests/test_oracle_*.py):
       bf16.*, linear.int_gemm (int64 brute force), linear.epilogue (float64 cross-check), moe.route_sort
-      (permutation properties), moe.combine (sequential bf16 sum restated two ways), layout.e8m0 map (closed form)
+      (permutation properties), moe.combine (sequential bf16 sum restated two ways), layout.e8m0 map (closed form),
+      linear.swiglu rounding structure (torch bf16, every gate pattern), moe.route (torch CPU ops, brute force),
+      linear.rmsnorm / rmsnorm_quant / res_norm_quant / swiglu_quant / headnorm / fullnorm STRUCTURE
+      (tests/test_oracle_norms.py: `w * bf16(x * inv)` against torch bf16 with wrong orders shown to differ, eps
+      inside the root, mean not sum, per-head slices and their weight vectors, whole-width statistics, head-major
+      outputs, untouched v, zero padding rows, fused kernels == composition of their parts), linear.row_sumsq
+      (every element counted once; within (log2 K + 4) half-ulps of math.fsum)
   parity unpinned (the arithmetic lives in MLX / mlx-lm, which are not vendored in the reference and not installed):
-      linear.swiglu (exp rounding), linear.rmsnorm_quant / rmsnorm reduction order, linear.headnorm, linear.fullnorm.
-      These follow the prose and kernel text of e2e/sc_kernels.py:120-160,317-328 with this build's own wave-64
-      reduction order; the kernels are held bit-exact to THIS restatement and within 1e-2 relative Frobenius error
-      of a float64 evaluation.
+      the ORDER of the FP32 additions inside the sum of squares (MLX: 32-lane simd_sum tree; here: 64-lane
+      butterfly) and metal::precise::rsqrt against IEEE 1/sqrt -- a few FP32 ulps of `inv`, which can flip a bf16
+      rounding of x * inv in rare elements; metal::precise::exp inside linear.swiglu (linear.exp_f32 rounds to the
+      same bf16 as the exact exponential for every bf16 input, so only a mis-rounding MLX exp could differ);
+      moe.route at exact probability ties (argpartition's choice) and MLX's softmax rounding at a bf16 tie.
+      No vector can settle these without MLX; the kernels are held bit-exact to THIS restatement and within 1e-2
+      relative Frobenius error of a float64 evaluation.
 """
