@@ -215,9 +215,9 @@ class DecodeQwen3:
     the o / down inputs inside those GEMVs' prologues; True: every quantization in a GEMV prologue; False: all
     separate.  graphs=True captures the two fixed-shape halves of every layer in HIP graphs on first use;
     graphs="step" captures the whole step (all layers and the output head) as one graph per cache.  A graph holds raw
-    pointers into the cache it was captured with, so the decoder keeps that cache object alive next to the graph and
-    re-captures when it is handed a different one; `release(cache)` drops the graphs (and the reference) of a cache
-    that is no longer needed.  Tensors returned by `step` are fresh in every mode (the graphs' static outputs are
+    pointers into the cache it was captured with, so the decoder keeps that cache object alive next to the graph and,
+    handed a different one, captures again IN PLACE of the old entries: at most one cache (the latest) and its graphs
+    are held, a fresh cache per prompt does not accumulate; `release(cache)` drops them before the next prompt.  Tensors returned by `step` are fresh in every mode (the graphs' static outputs are
     cloned).  fuse_attn=True (default): q/k norm, rotary embedding, cache append and the attention in one kernel;
     False: two kernels (same bits).  head="packed": the output projection quantized to the published SC-MXFP4 format
     (32-blocks, multipliers 1,2,4,8) whatever format the model's layers use."""
@@ -287,9 +287,11 @@ class DecodeQwen3:
 
     def _capture(self, key, fn, inputs, owner=None):
         """Capture fn(*static copies of inputs) once per (key, owner); returns (graph, static inputs, static outputs).
-        `owner` is the object whose memory the captured kernels point into (a cache or one of its layers): it is stored
-        with the graph, which keeps it alive (its id cannot be reused by a later object), and an entry captured for a
-        different owner is replaced."""
+        `owner` is the object whose memory the captured kernels point into (a cache or one of its layers).  A key
+        names a slot of the step ("step", ("pre", layer), ("post", layer)), never an object, and a slot holds the graph
+        of ONE owner: capturing for another cache replaces the entry, so the store keeps at most one cache (the most
+        recent one) and its graphs alive however many prompts come by, each with a fresh cache.  Alternating between
+        two live caches therefore re-captures at every switch; give each its own decoder."""
         if self._lookup(key, owner) is None:
             static = [t.clone() for t in inputs]
             s = torch.cuda.Stream()
@@ -304,8 +306,8 @@ class DecodeQwen3:
         return self.graphs[key]
 
     def _lookup(self, key, owner):
-        """The entry stored under key if it was captured for this very owner object; an entry of another owner (a key
-        built from the id of an object that has since been replaced) is dropped."""
+        """The entry stored under key if it was captured for this very owner object; an entry of another owner is
+        dropped (with its graph, static buffers and the reference that kept the old cache alive)."""
         entry = self.graphs.get(key)
         if entry is not None and entry[3] is not owner:
             del self.graphs[key]
@@ -356,7 +358,7 @@ class DecodeQwen3:
         if self.graphs is not None:
             self.pos.fill_(off)
         if self.whole_step:
-            out = self._replay(("step", id(cache)), lambda t: self._step_static(t, cache), [tok], owner=cache)
+            out = self._replay(("step",), lambda t: self._step_static(t, cache), [tok], owner=cache)
             for c in cache:
                 c.offset = off + 1
             return out.clone()     # the graph's static output is overwritten by the next replay
@@ -366,7 +368,7 @@ class DecodeQwen3:
             if self.graphs is None:
                 q = self._pre(h, nw, ws["qkv"], c, off)
             else:
-                q = self._replay(("pre", i, id(c)), lambda x, nw=nw, w=ws["qkv"], c=c: self._pre(x, nw, w, c, self.pos), [h],
+                q = self._replay(("pre", i), lambda x, nw=nw, w=ws["qkv"], c=c: self._pre(x, nw, w, c, self.pos), [h],
                                  owner=c)
             o = self._attn(c, q)
             if self.graphs is None:
