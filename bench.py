@@ -389,41 +389,55 @@ def main():
     if not a.no_decode:
         del sets, calls
         torch.cuda.empty_cache()
-        for name, n, k in DECODE:
-            bytes_call = n * k * (0.5 + 1.0 / 128) + 4 * n + 2 * k + 2 * n      # packed codes + 2-bit block codes + row
-            copies = max(2, -(-320 * 2 ** 20 // int(bytes_call)))              # scales + bf16 in / out
-            copies = min(copies, 160)
-            wsets = [tuple(up(t) for t in packed_random(rng, n, k)) for _ in range(copies)]
-            for batch in (1, 4):
-                x = up(acts(rng, batch, k)).to(torch.bfloat16)
-                out = torch.empty((batch, n), dtype=torch.bfloat16, device=dev)
-                argl = [(C.byref(fmt), x.data_ptr(), None, c.data_ptr(), b.data_ptr(), w.data_ptr(), None, out.data_ptr(),
-                         1, 1, None, C.c_float(0.0), batch, n, k, None, 0, 0, -1, sp) for c, b, w in wsets]
-                reps_d = max(copies, 100)
-                ms_d, ms_d_min = timeit(lambda i: check(lib.scmx_gemv(*argl[i % copies])), reps_d, reps=a.reps, warmup=copies,
-                                   warm_s=0.2)
-                us = ms_d * 1e3
-                # the same launches replayed from a HIP graph: kernel time without the host's per-call launch cost
-                ncap = min(copies, 40)
-                side = torch.cuda.Stream()
-                side.wait_stream(stream)
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, stream=side):
-                    ssp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-                    for i in range(ncap):
-                        check(lib.scmx_gemv(*(argl[i][:-1] + (ssp,))))
-                stream.wait_stream(side)
-                ms_g, _ = timeit(lambda i: graph.replay(), max(2, 100 // ncap), reps=a.reps, warm_s=0.1)
-                us_g = ms_g * 1e3 / ncap
-                bts = n * k * (0.5 + 1.0 / 128) + 4 * n + batch * (2 * k + 2 * n)
-                decode[f"{name}_b{batch}"] = {"us": round(us, 2), "us_min": round(ms_d_min * 1e3, 2),
-                                              "gbps": round(bts / us / 1e3, 1),
-                                              "pct_hbm": round(bts / us / 1e3 / PEAK_HBM_GBPS * 100, 1),
-                                              "us_graph": round(us_g, 2), "gbps_graph": round(bts / us_g / 1e3, 1),
-                                              "pct_hbm_graph": round(bts / us_g / 1e3 / PEAK_HBM_GBPS * 100, 1)}
-                del graph
-            del wsets
-            torch.cuda.empty_cache()
+        fmt_mx = pkg._lib.CFormat()
+        lib.scmx_mxfp4_format(C.byref(fmt_mx))
+
+        def mxfp4_random(n, k):
+            """A standard MXFP4 tensor read in place: random E2M1 nibbles, one E8M0 byte per 32-block (each row's bytes
+            within 3 of its lowest), and the row scales 2^(lowest - 128) the kernels place the blocks with."""
+            codes = rng.integers(0, 2 ** 32, n * k // 8, dtype=np.uint64).astype(np.uint32)
+            e8 = (rng.integers(0, 4, (n, k // 32)) + rng.integers(100, 120, (n, 1))).astype(np.uint8)
+            return codes, e8, np.exp2(e8.min(1).astype(np.float64) - 128).astype(np.float32)
+
+        # "" = the reference's own storage (2-bit block codes, e2e/sc_format.py:4-15); "_mxfp4" = BASELINE config 2's
+        # wording, nibbles + one E8M0 byte per 32-block, read in place
+        for form, cfmt, bc_bytes, gen in (("", fmt, 1.0 / 128, lambda n, k: packed_random(rng, n, k)),
+                                          ("_mxfp4", fmt_mx, 1.0 / 32, mxfp4_random)):
+            for name, n, k in DECODE:
+                bytes_call = n * k * (0.5 + bc_bytes) + 4 * n + 2 * k + 2 * n      # packed codes + block bytes + row
+                copies = max(2, -(-320 * 2 ** 20 // int(bytes_call)))              # scales + bf16 in / out
+                copies = min(copies, 160)
+                wsets = [tuple(up(t) for t in gen(n, k)) for _ in range(copies)]
+                for batch in (1, 4):
+                    x = up(acts(rng, batch, k)).to(torch.bfloat16)
+                    out = torch.empty((batch, n), dtype=torch.bfloat16, device=dev)
+                    argl = [(C.byref(cfmt), x.data_ptr(), None, c.data_ptr(), b.data_ptr(), w.data_ptr(), None, out.data_ptr(),
+                             1, 1, None, C.c_float(0.0), batch, n, k, None, 0, 0, -1, sp) for c, b, w in wsets]
+                    reps_d = max(copies, 100)
+                    ms_d, ms_d_min = timeit(lambda i: check(lib.scmx_gemv(*argl[i % copies])), reps_d, reps=a.reps, warmup=copies,
+                                       warm_s=0.2)
+                    us = ms_d * 1e3
+                    # the same launches replayed from a HIP graph: kernel time without the host's per-call launch cost
+                    ncap = min(copies, 40)
+                    side = torch.cuda.Stream()
+                    side.wait_stream(stream)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        ssp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                        for i in range(ncap):
+                            check(lib.scmx_gemv(*(argl[i][:-1] + (ssp,))))
+                    stream.wait_stream(side)
+                    ms_g, _ = timeit(lambda i: graph.replay(), max(2, 100 // ncap), reps=a.reps, warm_s=0.1)
+                    us_g = ms_g * 1e3 / ncap
+                    bts = n * k * (0.5 + bc_bytes) + 4 * n + batch * (2 * k + 2 * n)
+                    decode[f"{name}_b{batch}{form}"] = {"us": round(us, 2), "us_min": round(ms_d_min * 1e3, 2),
+                                                  "gbps": round(bts / us / 1e3, 1),
+                                                  "pct_hbm": round(bts / us / 1e3 / PEAK_HBM_GBPS * 100, 1),
+                                                  "us_graph": round(us_g, 2), "gbps_graph": round(bts / us_g / 1e3, 1),
+                                                  "pct_hbm_graph": round(bts / us_g / 1e3 / PEAK_HBM_GBPS * 100, 1)}
+                    del graph
+                del wsets
+                torch.cuda.empty_cache()
 
     # ---- offline quantizer on the device: float32 weights -> packed SC-MXFP4 -----------------------------------
     quant = {}

@@ -54,6 +54,14 @@ const char* scmx_last_error(void);
  * (sc_format.DEFAULT, e2e/sc_format.py:63). */
 void scmx_default_format(scmx_format* f);
 
+/* Fill `f` with the descriptor of a STANDARD MXFP4 tensor read in place (block 32, bc_bits 8, n_mult 0): `codes` are the
+ * tensor's E2M1 nibble bytes (two codes per byte, even k low), `bcodes` its E8M0 scale bytes [N, K/32], one per
+ * 32-block, exactly as e2e/fused_qwen38.py:319-334 lays them out; `wscale` [N] = 2^(lowest exponent byte of the row -
+ * 128), which scmx_mxfp4_to_sc writes (with bcodes = NULL it writes nothing else).  A block decodes with shift = byte -
+ * lowest, so a row's bytes must lie in 1..254 and span at most 3 (scmx_mxfp4_to_sc reports otherwise).  Accepted by
+ * scmx_gemv, scmx_mm_w4a8, scmx_linear_w4a8(_static) and scmx_moe_mm; scmx_unpack_i8 takes the converted form only. */
+void scmx_mxfp4_format(scmx_format* f);
+
 /* ---- dense prefill ------------------------------------------------------------------------------------------ */
 
 /* Packed weights -> INT8 [n_rows, K].  Replaces unpack_i8, e2e/sc_kernels.py:34-50,480-483 (and unpack_experts,
@@ -239,7 +247,10 @@ int scmx_rot_quant(const uint16_t* x, const float* signs, int8_t* xq, float* xs,
 
 /* Standard MXFP4 rows (E2M1 nibbles + one E8M0 byte per 32-block, e8m0 [N, K/32]) -> block codes and row scales of
  * the default format: shift = e8m0 - min over the row, wscale = 2^(min - 128).  The nibble bytes are used as the
- * code words unchanged.  status[0] is set to 1 when some row's exponents span more than 3 (not INT8-embeddable).
+ * code words unchanged.  status[0] (cleared by the caller) gets bit 0 set when some row's exponents span more than 3 (not
+ * INT8-embeddable) and bit 1 when a row holds the bytes 0 or 255 (fine for the converted form, not for reading the
+ * tensor in place).  bcodes may
+ * be NULL: then only the row scales are written, which is all that the in-place form (scmx_mxfp4_format) needs.
  * Device form of the map in e2e/fused_qwen38.py:319-334 (inverse direction) and e2e/gptq_pack.py:29-47. */
 int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,
                      void* stream);

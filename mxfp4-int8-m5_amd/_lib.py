@@ -22,6 +22,7 @@ SIGNATURES = {
     "scmx_version": (C.c_char_p, []),
     "scmx_last_error": (C.c_char_p, []),
     "scmx_default_format": (None, [_FMT]),
+    "scmx_mxfp4_format": (None, [_FMT]),
     "scmx_unpack_i8": (_I, [_FMT, _P, _P, _P, _L, _L, _P]),
     "scmx_act_quant": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "scmx_mm_i8_i32": (_I, [_P, _P, _P, _I, _I, _I, _P]),

@@ -51,6 +51,26 @@ int make_dev_format(const scmx_format* f, DevFormat* out) {
         set_error("format: block %d not in {8,16,32,64,128}", b);
         return SCMX_ERR_FORMAT;
     }
+    if (b == 32 && f->bc_bits == 8 && f->n_mult == 0) {   // standard MXFP4: E8M0 bytes in place of block codes
+        const int mag[8] = {0, 1, 2, 3, 4, 6, 8, 12};
+        for (int i = 0; i < 8; ++i)
+            if (f->code_mag[i] != mag[i]) {
+                set_error("format: the E8M0 form takes the E2M1 code magnitudes 0,1,2,3,4,6,8,12");
+                return SCMX_ERR_FORMAT;
+            }
+        DevFormat d;
+        memset(&d, 0, sizeof(d));
+        d.lut_lo = 0x03020100u;
+        d.lut_hi = 0x0C080604u;
+        d.mult[0] = 0x08040201u;
+        d.block = 32;
+        d.block_log2 = 5;
+        d.bc_bits = 8;
+        d.pow2 = 1;
+        d.e8m0 = 1;
+        *out = d;
+        return SCMX_OK;
+    }
     if (!(f->bc_bits == 1 || f->bc_bits == 2 || f->bc_bits == 4 || f->bc_bits == 8) || f->n_mult < 1 ||
         f->n_mult > 16 || f->n_mult > (1 << f->bc_bits)) {
         set_error("format: bc_bits %d / n_mult %d unsupported (need bc_bits in {1,2,4,8}, n_mult <= min(16, 2^bc_bits))",
@@ -299,8 +319,10 @@ __global__ __launch_bounds__(256) void mxfp4_to_sc_kernel(const uint8_t* __restr
         lo = min(lo, __shfl_xor(lo, off, WAVE));
         hi = max(hi, __shfl_xor(hi, off, WAVE));
     }
-    if (hi - lo > 3 && lane == 0) status[0] = 1;
-    for (int byte = lane; byte < nb / 4; byte += 64) {
+    if (hi - lo > 3 && lane == 0) atomicOr(status, 1);
+    // exponent bytes 0 (a scale below every normal float's) and 255 (NaN in the MX specification) cannot be read in place
+    if ((lo < 1 || hi > 254) && lane == 0) atomicOr(status, 2);
+    for (int byte = lane; bcodes && byte < nb / 4; byte += 64) {
         uint32_t v = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) v |= (uint32_t(min(int(e[4 * byte + j]) - lo, 3))) << (2 * j);
@@ -323,6 +345,13 @@ extern "C" {
 const char* scmx_version(void) { return "scmx 0.2 (gfx950) " SCMX_BUILD_ID; }
 const char* scmx_last_error(void) { return g_err; }
 
+void scmx_mxfp4_format(scmx_format* f) {
+    scmx_default_format(f);
+    f->bc_bits = 8;
+    f->n_mult = 0;
+    for (int i = 0; i < 16; ++i) f->mult[i] = 0;
+}
+
 void scmx_default_format(scmx_format* f) {
     memset(f, 0, sizeof(*f));
     f->block = 32;
@@ -337,6 +366,10 @@ int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t*
                    int64_t K, void* stream) {
     DevFormat f;
     if (int rc = make_dev_format(fmt, &f)) return rc;
+    if (f.e8m0) {
+        set_error("unpack_i8: the E8M0 form needs the row scales to place a block; convert with scmx_mxfp4_to_sc first");
+        return SCMX_ERR_FORMAT;
+    }
     if (!codes || !bcodes || !wq || n_rows < 0 || K <= 0 || K % f.block || (K / f.block * f.bc_bits) % 8) {
         set_error("unpack_i8: need non-null pointers, K (%lld) a multiple of block %d and whole block-code bytes per row",
                   (long long)K, f.block);
@@ -403,7 +436,7 @@ int scmx_rot_quant(const uint16_t* x, const float* signs, int8_t* xq, float* xs,
 
 int scmx_mxfp4_to_sc(const uint8_t* e8m0, uint8_t* bcodes, float* wscale, int32_t* status, int64_t N, int64_t K,
                      void* stream) {
-    if (!e8m0 || !bcodes || !wscale || !status || N < 0 || N > (int64_t(1) << 32) || K <= 0 || K % 128 || K > (int64_t(1) << 30)) {
+    if (!e8m0 || !wscale || !status || N < 0 || N > (int64_t(1) << 32) || K <= 0 || K % 128 || K > (int64_t(1) << 30)) {
         set_error("mxfp4_to_sc: need non-null pointers, N <= 2^32 and K %% 128 == 0, K <= 2^30 (K = %lld)", (long long)K);
         return SCMX_ERR_ARG;
     }

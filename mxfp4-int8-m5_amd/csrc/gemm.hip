@@ -39,7 +39,9 @@ struct GemmArgs {
 // with the FP4 conversion); B_PACKED_B16M: that codebook on 16-element blocks with 4-bit codes for consecutive integer
 // multipliers (FP4 conversion, then one fused multiply-add); B_PACKED_GENERIC: any member of the format family (table
 // decode).
-enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3, B_PACKED_B16M = 4 };
+// B_PACKED_E8M0: a standard MXFP4 tensor in place -- B_PACKED_DEFAULT's decode with the block's shift taken from its
+// E8M0 byte minus the row's lowest one (which the row scale carries).
+enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3, B_PACKED_B16M = 4, B_PACKED_E8M0 = 5 };
 
 // FD = number of fragment register buffers: fragments are fetched FD - 1 k slices ahead of their MFMAs.
 // SKIP (grouped launches): a row tile that ends inside its expert's segment multiplies only the 32-row blocks that hold
@@ -161,6 +163,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         a_dst[j] = swz(row, kc);
     }
     int b_src[B_PER], b_bc[B_PER], b_dst[B_PER], b_dst2[B_PER], b_k[B_PER];
+    [[maybe_unused]] uint32_t b_rmin[B_PER];   // B_PACKED_E8M0: lowest exponent byte of the thread's weight row
 #pragma unroll
     for (int j = 0; j < B_PER; ++j) {
         const int c = tid + j * NT;
@@ -181,7 +184,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             // (two 4-bit codes per byte: 32)
             b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16    ? (kb * 8 * WPC) >> 6
                                              : BMODE == B_PACKED_B16M ? (kb * 8 * WPC) >> 5
+                                             : BMODE == B_PACKED_E8M0 ? (kb * 8 * WPC) >> 5
                                                                       : 0);
+            if (BMODE == B_PACKED_E8M0) b_rmin[j] = e8m0_row_min(a.wscale[erow + gn]);
             if (PK) {   // the run's 16 code bytes as they are
                 b_dst[j] = BM * BK + swzp(row, kb);
                 b_dst2[j] = 0;
@@ -239,6 +244,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                         r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 6, 0);
                     if (BMODE == B_PACKED_B16M)      // 16-blocks, 4-bit codes: 32 weights
                         r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 5, 0);
+                    if (BMODE == B_PACKED_E8M0)      // one exponent byte per 32 weights
+                        r.bc[j] = __builtin_amdgcn_raw_buffer_load_b8(rbc, b_bc[j], k0 >> 5, 0);
                 }
             }
     };
@@ -270,6 +277,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
                         if (BMODE == B_PACKED_DEFAULT) {
                             const uint32_t blk = uint32_t(k0 + b_k[j]) >> 5;
                             decode_word_fp4(r.b[j][w], fp4_scale((uint32_t(r.bc[j]) >> (2 * (blk & 3))) & 3u), o[j][2 * w],
+                                            o[j][2 * w + 1]);
+                        } else if (BMODE == B_PACKED_E8M0) {   // the run lies inside one block
+                            decode_word_fp4(r.b[j][w], fp4_scale((uint32_t(r.bc[j]) - b_rmin[j]) & 0x7Fu), o[j][2 * w],
                                             o[j][2 * w + 1]);
                         } else if (BMODE == B_PACKED_B16) {
                             const uint32_t blk = uint32_t(k0 + b_k[j] + 8 * w) >> 4;
@@ -693,13 +703,16 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16M)
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+        else if (bmode == B_PACKED_E8M0)
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
         else
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
     }
 }
 
 static int packed_mode(const DevFormat& f) {
-    return is_default_format(f)        ? B_PACKED_DEFAULT
+    return is_mxfp4_e8m0_format(f)     ? B_PACKED_E8M0
+           : is_default_format(f)      ? B_PACKED_DEFAULT
            : is_pow2_block16_format(f) ? B_PACKED_B16
            : is_block16_range_format(f) ? B_PACKED_B16M
                                         : B_PACKED_GENERIC;
@@ -793,6 +806,10 @@ int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, 
     if (int rc = check_gemm_common("mm_w4a8", M, N, K, epi, true, xq, xscale, wscale, res, out)) return rc;
     if (!codes || !bcodes || uintptr_t(codes) % 16 || K % f.block || (K / f.block * f.bc_bits) % 8) {
         set_error("mm_w4a8: codes must be 16-byte aligned, K a multiple of the block with whole block-code bytes per row");
+        return SCMX_ERR_ARG;
+    }
+    if (f.e8m0 && !wscale) {
+        set_error("mm_w4a8: the E8M0 form decodes with the row scales; wscale must not be NULL");
         return SCMX_ERR_ARG;
     }
     if (M == 0) return SCMX_OK;
@@ -933,6 +950,10 @@ int scmx_moe_mm(const scmx_format* fmt, const int8_t* xq, const float* xscale, c
         return rc;
     if (!codes || !bcodes || uintptr_t(codes) % 16 || K % f.block || (K / f.block * f.bc_bits) % 8) {
         set_error("moe_mm: codes must be 16-byte aligned, K a multiple of the block with whole block-code bytes per row");
+        return SCMX_ERR_ARG;
+    }
+    if (f.e8m0 && !wscale) {
+        set_error("moe_mm: the E8M0 form decodes with the row scales; wscale must not be NULL");
         return SCMX_ERR_ARG;
     }
     if (R == 0) return SCMX_OK;

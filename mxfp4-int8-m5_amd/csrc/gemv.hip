@@ -404,6 +404,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     constexpr bool FP4 = MODE >= 2;
     constexpr bool B16 = MODE == 3;
     constexpr bool B16M = MODE == 4;
+    // 5: a standard MXFP4 tensor in place -- the FP4 conversion with one E8M0 byte per 32-block instead of a 2-bit code
+    constexpr bool E8 = MODE == 5;
     constexpr int XB = FP4 ? 2 : 1;                    // bytes per staged activation
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int K = a.K, N = a.N;
@@ -431,6 +433,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     struct Item {
         u32x4 w[R];
         uint32_t bc[R];
+        uint32_t rmin[E8 ? R : 1];   // E8: the rows' lowest exponent bytes (from their scales; wave-uniform)
     };
     const int g_stride = gridDim.x * (NT / 64);
     const int CI = (nchunk + 63) / 64;                 // items per row group
@@ -449,7 +452,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
         for (int r = 0; r < R; ++r) {
             it.w[r] = __builtin_amdgcn_raw_buffer_load_b128(rc, int(16u * cc), r * (K / 2), W_STREAM);
             // the byte with the chunk's block codes: 4 blocks per byte = 4 chunks of 32 weights, or 2 with 16-blocks
-            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> (B16M ? 0 : B16 ? 1 : 2)), r * a.bc_row_bytes, 0);
+            if (DEFAULT_FMT) it.bc[r] = __builtin_amdgcn_raw_buffer_load_b8(rb, int(cc >> ((B16M || E8) ? 0 : B16 ? 1 : 2)), r * a.bc_row_bytes, 0);
+            if constexpr (E8) it.rmin[E8 ? r : 0] = e8m0_row_min(a.wscale[erow + size_t(g) * R + r]);
         }
     };
     auto compute_item = [&](const Item& it, int g, uint32_t c_in, int (&acc)[NV]) {
@@ -468,6 +472,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
                     scale[r][0] = scale[r][1] = 2.0f;
 #pragma unroll
                     for (int b = 0; b < BATCH; ++b) part2[r][b] = 0.0f;
+                } else if (E8) {
+                    scale[r][0] = scale[r][1] = __uint_as_float(((128u + bc[r] - it.rmin[E8 ? r : 0]) & 0xFFu) << 23);
                 } else if (B16) {
                     scale[r][0] = __uint_as_float((128u + ((bc[r] >> (4 * (c & 1))) & 3u)) << 23);
                     scale[r][1] = __uint_as_float((128u + ((bc[r] >> (4 * (c & 1) + 2)) & 3u)) << 23);
@@ -837,8 +843,9 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 // SPLIT (narrow layers): one row group per workgroup, the waves take the 512-wide pieces of K in turn (wave, wave + 4, ...)
 // and their INT32 partial totals meet in LDS: the layer's few rows are spread over 4 x N / 16 waves with one or a few
 // pieces each instead of N / 16 waves walking all of K.
-template <int BATCH, int POL, bool SPLIT, int WAVE_PRE>
-__global__ __launch_bounds__(256) void gemv_hmfma_kernel(const GemvArgs a) {
+// E8: a standard MXFP4 tensor in place -- the piece's 16 blocks bring 16 E8M0 bytes per row instead of 4 code bytes.
+template <int BATCH, int POL, bool SPLIT, int WAVE_PRE, bool E8 = false>
+__global__ __launch_bounds__(256, (E8 && WAVE_PRE <= 4) ? 4 : 1) void gemv_hmfma_kernel(const GemvArgs a) {
     constexpr int NT = 256;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int K = a.K, N = a.N;
@@ -859,10 +866,20 @@ __global__ __launch_bounds__(256) void gemv_hmfma_kernel(const GemvArgs a) {
     const int CI = Kp / 512;                           // pieces per row group
     const int g_stride = gridDim.x * (NT / 64);
     const int brow = r < BATCH ? r : 0;                // the batch row this lane's MFMA column reads
+    // E8, wide layers (E8T; at least 3 pieces per row group): a row group's exponent bytes, 16 rows x K / 32, are at most
+    // 1 KiB -- ONE wave-wide 16-byte load per row group instead of a strided 4-byte load per piece (whose 16 cache lines per
+    // instruction cost the batch-4 output head a quarter of its rate).  They wait in registers (`e8n`) until the group's
+    // first piece is multiplied, then sit in a wave-private LDS tile of 16 rows x 80 bytes (conflict-free 4-byte reads).
+    constexpr bool E8T = E8 && !SPLIT;
+    constexpr int EPITCH = 80;
+    int8_t* e8tile = reinterpret_cast<int8_t*>(sxs + ((BATCH + 3) & ~3)) + size_t(NT / 64) * 16 * WPITCH + size_t(wave) * 16 * EPITCH;
+    [[maybe_unused]] u32x4 e8n = u32x4{0u, 0u, 0u, 0u};
+    [[maybe_unused]] uint32_t rmin_next = 0, rmin_cur = 0;
 
     struct Item {
         u32x4 w[4];     // loads i = 0..3 of the piece: the 32-weight block 4 i + c of row r
         uint32_t bc;    // the piece's four block-code bytes of row r (byte i: blocks 4 i .. 4 i + 3)
+        uint32_t rmin;  // E8: the row's lowest exponent byte (bc then holds the exponent bytes of blocks 4 c .. 4 c + 3)
     };
     const auto load_item = [&](Item& it, int g, int ci) {
         const uint8_t* crow = reinterpret_cast<const uint8_t*>(a.codes) + size_t(g) * 16 * (K / 2);   // uniform
@@ -874,7 +891,17 @@ __global__ __launch_bounds__(256) void gemv_hmfma_kernel(const GemvArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)   // rows 4 i .. 4 i + 3: lane l reads 16 bytes at byte 16 (l % 16) of row 4 i + l / 16
             it.w[i] = __builtin_amdgcn_raw_buffer_load_b128(rc, (4 * i + c) * (K / 2) + 16 * r, ci * 256, POL);
-        it.bc = __builtin_amdgcn_raw_buffer_load_b32(rb, r * a.bc_row_bytes, ci * 4, 0);
+        if constexpr (E8T) {
+            if (ci == 0) {   // the first piece of a row group brings the group's exponent bytes and lowest exponents
+                e8n = __builtin_amdgcn_raw_buffer_load_b128(rb, r * a.bc_row_bytes + 16 * c, 0, 0);
+                rmin_next = e8m0_row_min(a.wscale[size_t(g) * 16 + r]);
+            }
+        } else if constexpr (E8) {
+            it.bc = __builtin_amdgcn_raw_buffer_load_b32(rb, r * a.bc_row_bytes + 4 * c, ci * 16, 0);
+            it.rmin = e8m0_row_min(a.wscale[size_t(g) * 16 + r]);
+        } else {
+            it.bc = __builtin_amdgcn_raw_buffer_load_b32(rb, r * a.bc_row_bytes, ci * 4, 0);
+        }
     };
     f4 acc0, acc1;     // two chains: consecutive MFMAs do not wait for each other
     int tot[4];
@@ -883,16 +910,29 @@ __global__ __launch_bounds__(256) void gemv_hmfma_kernel(const GemvArgs a) {
         for (int i = 0; i < 4; ++i) tot[i] += int(acc0[i]) + int(acc1[i]);
         acc0 = acc1 = f4{0.0f, 0.0f, 0.0f, 0.0f};
     };
+    // Which of the piece's 16 blocks a lane multiplies is free (the MFMA sums over the four lane groups): group c takes
+    // blocks 4 i + c, or with E8M0 bytes blocks 4 c + i, whose four exponent bytes are one aligned 4-byte load.
     const auto compute_item = [&](const Item& it, int ci) {
-        const int8_t* xrow = sx + size_t(brow) * pitch + (size_t(ci) * 512 + 32 * c) * 2;
+        const int8_t* xrow = sx + size_t(brow) * pitch + (size_t(ci) * 512 + (E8 ? 128 : 32) * c) * 2;
 #pragma unroll
         for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(slot + (4 * i + c) * WPITCH + 16 * r) = it.w[i];
-        u32x4 wt[4];   // row r, blocks 4 i + c: bytes 64 i + 16 c of the row's 256
+        u32x4 wt[4];   // row r, blocks 4 i + c (E8: 4 c + i): bytes 64 i + 16 c (64 c + 16 i) of the row's 256
 #pragma unroll
-        for (int i = 0; i < 4; ++i) wt[i] = *reinterpret_cast<const u32x4*>(slot + r * WPITCH + 64 * i + 16 * c);
+        for (int i = 0; i < 4; ++i)
+            wt[i] = *reinterpret_cast<const u32x4*>(slot + r * WPITCH + (E8 ? 64 * c + 16 * i : 64 * i + 16 * c));
+        uint32_t ebytes = it.bc, elow = it.rmin;
+        if constexpr (E8T) {
+            if (ci == 0) {
+                *reinterpret_cast<u32x4*>(e8tile + r * EPITCH + 16 * c) = e8n;
+                rmin_cur = rmin_next;
+            }
+            ebytes = *reinterpret_cast<const uint32_t*>(e8tile + r * EPITCH + 16 * ci + 4 * c);   // blocks 4 c .. 4 c + 3 of the piece
+            elow = rmin_cur;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float scale = fp4_scale((it.bc >> (8 * i + 2 * c)) & 3u);
+            const float scale = E8 ? fp4_scale((((ebytes >> (8 * i)) & 0xFFu) - elow) & 0x7Fu)
+                                   : fp4_scale((it.bc >> (8 * i + 2 * c)) & 3u);
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 const uint32_t w = wt[i][d];
@@ -901,7 +941,7 @@ __global__ __launch_bounds__(256) void gemv_hmfma_kernel(const GemvArgs a) {
                 const h2 q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 2);
                 const h2 q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 3);
                 const h8 wv = h8{q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
-                const h8 xv = *reinterpret_cast<const h8*>(xrow + (128 * i + 8 * d) * 2);
+                const h8 xv = *reinterpret_cast<const h8*>(xrow + ((E8 ? 32 : 128) * i + 8 * d) * 2);
                 if (d & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xv, acc1, 0, 0, 0);
                 else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xv, acc0, 0, 0, 0);
             }
@@ -1038,14 +1078,16 @@ static void launch_gemv(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
     // more rows sharing the weight stream its extra LDS reads cost more than the integer dot products
     // dflt: 1 = the published format, 2 = its 16-block variant (fast path for one activation row only), 0 = other
     // 3 = the 16-block family members with consecutive integer multipliers (likewise)
-    const int mode = dflt == 1 ? (BATCH == 1 ? 2 : 1) : (dflt >= 2 && BATCH == 1) ? dflt + 1 : 0;
+    // 4 = a standard MXFP4 tensor in place (E8M0 bytes; the FP4-conversion path whatever the batch)
+    const int mode = dflt == 4 ? 5 : dflt == 1 ? (BATCH == 1 ? 2 : 1) : (dflt >= 2 && BATCH == 1) ? dflt + 1 : 0;
     const size_t smem = size_t(BATCH) * ((a.K + 2047) & ~2047) * (mode >= 2 ? 2 : 1) + (68 + BATCH) * sizeof(float);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024)
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
         kernel<<<grid, block, smem, s>>>(a);
     };
-    if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
+    if (mode == 5) go(gemv_kernel<BATCH, R, 5>);
+    else if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
     else if (mode == 3) go(gemv_kernel<BATCH, R, 3>);
     else if (mode == 4) go(gemv_kernel<BATCH, R, 4>);
     else if (mode == 1) go(gemv_kernel<BATCH, R, 1>);
@@ -1065,28 +1107,35 @@ static void launch_gemv_mfma(const GemvArgs& a, hipStream_t s) {
     gemv_mfma_kernel<BATCH><<<grid, block, smem, s>>>(a);
 }
 
-template <int BATCH>
+template <int BATCH, bool E8 = false>
 static void launch_gemv_hmfma(const GemvArgs& a, bool split, hipStream_t s) {
     const int groups = a.N / 16;
     const int want = (groups + 3) / 4;
     const int rounds = (want + 1535) / 1536;   // 6 waves per SIMD are resident
     const dim3 grid(split ? groups : (want + rounds - 1) / rounds), block(256);
-    const size_t smem = size_t(BATCH) * (((a.K + 511) & ~511) * 2 + 16) + (68 + ((BATCH + 3) & ~3)) * sizeof(float) + 4 * 16 * 272;
+    const size_t smem = size_t(BATCH) * (((a.K + 511) & ~511) * 2 + 16) + (68 + ((BATCH + 3) & ~3)) * sizeof(float) + 4 * 16 * 272 +
+                        (E8 ? 4 * 16 * 80 : 0);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024)
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
         kernel<<<grid, block, smem, s>>>(a);
     };
     // the early request of the activation rows holds K / 512 chunks per lane: 4 for K <= 2048, 12 up to 6144
-    if (!split) go(gemv_hmfma_kernel<BATCH, W_STREAM, false, 4>);
-    else if (a.K <= 2048) go(gemv_hmfma_kernel<BATCH, W_STREAM, true, 4>);
-    else go(gemv_hmfma_kernel<BATCH, W_STREAM, true, 12>);
+    if (!split) go(gemv_hmfma_kernel<BATCH, W_STREAM, false, 4, E8>);
+    else if (a.K <= 2048) go(gemv_hmfma_kernel<BATCH, W_STREAM, true, 4, E8>);
+    else go(gemv_hmfma_kernel<BATCH, W_STREAM, true, 12, E8>);
 }
 
 template <int BATCH>
 static void launch_gemv_rows(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
     // wide layers in the published format: half-precision MFMA dot products (whole row groups of 16, pieces of 512)
     // (several activation rows, K up to 2048: beyond that its half-precision activations cost too much LDS)
+    if (BATCH > 1 && dflt == 4 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 8192 && size_t(BATCH) * a.K <= 32768 &&
+        uintptr_t(a.bcodes) % 4 == 0) {   // the same two kernels reading E8M0 bytes (4 per lane and piece, one aligned load)
+        // wide layers: the form that loads a row group's exponent bytes at once needs 3 pieces per group (K >= 1536)
+        if (a.N >= HMFMA_MIN_ROWS && a.K <= 2048 && a.K >= 1536) return launch_gemv_hmfma<BATCH, true>(a, false, s);
+        return launch_gemv_hmfma<BATCH, true>(a, true, s);
+    }
     if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 2048 && a.N >= HMFMA_MIN_ROWS)
         return launch_gemv_hmfma<BATCH>(a, false, s);
     // narrow layers with several activation rows: the same kernel with K split over the waves of a workgroup
@@ -1160,7 +1209,11 @@ extern "C" int scmx_gemv(const scmx_format* fmt, const void* x, const float* xsc
     a.bc_row_bytes = K / f.block * f.bc_bits / 8;
     a.eidx = eidx; a.n_eidx = n_eidx; a.xstride = xstride; a.shared_expert = eidx ? shared_expert : -1;
     a.fmt = f;
-    const int dflt = is_default_format(f) ? 1 : is_pow2_block16_format(f) ? 2 : is_block16_range_format(f) ? 3 : 0;
+    const int dflt = is_mxfp4_e8m0_format(f)    ? 4
+                     : is_default_format(f)       ? 1
+                     : is_pow2_block16_format(f)  ? 2
+                     : is_block16_range_format(f) ? 3
+                                                  : 0;
     hipStream_t s = (hipStream_t)stream;
     switch (batch) {
         case 1: launch_gemv_rows<1>(a, slots, dflt, s); break;

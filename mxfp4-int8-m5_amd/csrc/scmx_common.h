@@ -25,6 +25,7 @@ struct DevFormat {
     int32_t block_log2;
     int32_t bc_bits;    // 1, 2, 4 or 8
     int32_t pow2;
+    int32_t e8m0;       // 1: the block-code bytes are E8M0 exponents of a standard MXFP4 tensor (block 32, bc_bits 8)
 };
 
 // Host: validate a caller's format and build the device view.  Returns 0 or SCMX_ERR_FORMAT.
@@ -51,6 +52,10 @@ inline bool is_block16_range_format(const DevFormat& d) {
     }
     return m0 >= 1;
 }
+
+// Standard MXFP4 read in place: one E8M0 byte per 32-block instead of a block code.  A row's lowest exponent is
+// carried by its scale, wscale = 2^(lowest - 128), so the block's shift is byte - (exponent field of wscale + 1).
+inline bool is_mxfp4_e8m0_format(const DevFormat& d) { return d.e8m0 != 0; }
 
 // Compute units of the current device (queried once per device).
 int device_cus();
@@ -168,6 +173,8 @@ __device__ __forceinline__ void decode_word_split(uint32_t w, const BlockLut& t,
 // byte of each half is q in two's complement; one byte permute gathers four of them.
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float fp4_scale(uint32_t shift) { return __uint_as_float((128u + shift) << 23); }
+// Lowest E8M0 exponent of a row of a standard MXFP4 tensor, recovered from its scale 2^(lowest - 128) (lowest >= 1).
+__device__ __forceinline__ uint32_t e8m0_row_min(float wscale) { return ((__float_as_uint(wscale) >> 23) & 0xFFu) + 1u; }
 __device__ __forceinline__ void decode_word_fp4(uint32_t w, float scale, uint32_t& a, uint32_t& b) {
     const half2_t bias = half2_t{_Float16(1536.0f), _Float16(1536.0f)};
     const half2_t q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 0) + bias;

@@ -25,8 +25,16 @@ class Format:
 
     def __post_init__(self):
         assert self.block % 8 == 0, "one code word (8 weights) must lie in one block"
+        if not self.mult:   # MXFP4: the block bytes are E8M0 exponents, the multiplier is 2^(byte - the row's lowest)
+            assert self.block == 32 and self.bc_bits == 8 and tuple(self.code_mag) == (0, 1, 2, 3, 4, 6, 8, 12)
+            return
         assert self.bc_bits in (1, 2, 4, 8) and len(self.mult) <= 2 ** self.bc_bits
         assert len(self.code_mag) == 8 and max(self.code_mag) * max(self.mult) <= 127, "must fit INT8"
+
+    @property
+    def e8m0(self):
+        """True for a standard MXFP4 tensor read in place (`MXFP4` below)."""
+        return not self.mult
 
     @property
     def per_byte(self):
@@ -49,6 +57,10 @@ class Format:
 
 
 DEFAULT = Format()
+# A standard MXFP4 tensor read in place (e2e/fused_qwen38.py:319-334): `codes` = its E2M1 nibble bytes, `bcodes` = its
+# E8M0 bytes uint8 [N, K/32], `wscale` = mxfp4_row_scales(e8m0).  Taken by gemv, mm_epi / linear_w4a8 on a PackedWq,
+# and moe_mm; 4.25 bits per weight + 32 / K.
+MXFP4 = Format(block=32, mult=(), bc_bits=8)
 
 
 def _pack_bcodes(bcode, fmt):
@@ -117,9 +129,30 @@ def from_mxfp4(nibbles, e8m0):
     ws = torch.empty(n, dtype=torch.float32, device=e8m0.device)
     status = torch.zeros(1, dtype=torch.int32, device=e8m0.device)
     _lib.call("scmx_mxfp4_to_sc", _lib.ptr(e8m0), _lib.ptr(bc), _lib.ptr(ws), _lib.ptr(status), n, k, _lib.stream())
-    if int(status.item()):
+    if int(status.item()) & 1:
         raise ValueError("a row's block exponents span more than 3: not INT8-embeddable")
     return nibbles.contiguous().view(torch.int32).reshape(-1), bc, ws
+
+
+def mxfp4_row_scales(e8m0):
+    """The row scales that let the kernels read a standard MXFP4 tensor in place (fmt=MXFP4): wscale [N] =
+    2^(lowest E8M0 byte of the row - 128).  Raises if a row's exponents span more than 3 or hold the bytes 0 / 255."""
+    n, nb = e8m0.shape
+    assert e8m0.dtype == torch.uint8
+    ws = torch.empty(n, dtype=torch.float32, device=e8m0.device)
+    status = torch.zeros(1, dtype=torch.int32, device=e8m0.device)
+    _lib.call("scmx_mxfp4_to_sc", _lib.ptr(e8m0), None, _lib.ptr(ws), _lib.ptr(status), n, nb * 32, _lib.stream())
+    st = int(status.item())
+    if st & 1:
+        raise ValueError("a row's block exponents span more than 3: not INT8-embeddable")
+    if st & 2:
+        raise ValueError("exponent bytes 0 and 255 cannot be read in place; convert with from_mxfp4")
+    return ws
+
+
+def mxfp4_codes(nibbles):
+    """The nibble bytes of a standard MXFP4 tensor [N, K/2] as the kernels' code words (a view, no copy)."""
+    return nibbles.contiguous().view(torch.int32).reshape(-1)
 
 
 def quantize(w, fmt=None, with_q=True):

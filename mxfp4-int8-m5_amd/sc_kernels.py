@@ -40,8 +40,9 @@ def _check_dtype(dtype):
 class PackedWq:
     """Packed weights standing in for the INT8 tensor unpack_i8 would produce."""
 
-    def __init__(self, codes, bcodes, N, K, fmt):
+    def __init__(self, codes, bcodes, N, K, fmt, wscale=None):
         self.codes, self.bcodes, self.N, self.K, self.fmt = codes, bcodes, N, K, fmt
+        self.wscale = wscale   # a standard MXFP4 tensor read in place decodes with its row scales (F.MXFP4)
         self.shape, self.dtype, self.device = (N, K), torch.int8, codes.device
 
     def materialize(self):
@@ -54,11 +55,14 @@ class PackedWq:
         return self.materialize().cpu()
 
 
-def unpack_i8(codes, bcodes, N, K, deps=(), lazy=None, fmt=None):
-    """Packed codes (flat, 4-byte ints) + block codes uint8 [N, ..] -> INT8 [N, K]."""
+def unpack_i8(codes, bcodes, N, K, deps=(), lazy=None, fmt=None, wscale=None):
+    """Packed codes (flat, 4-byte ints) + block codes uint8 [N, ..] -> INT8 [N, K].  fmt=F.MXFP4 (E8M0 bytes as block
+    codes) exists as the lazy handle only and takes the row scales along (F.mxfp4_row_scales)."""
     fmt = fmt or F.DEFAULT
+    if fmt.e8m0 and wscale is None:
+        raise ValueError("the MXFP4 form decodes with its row scales: pass wscale=sc_format.mxfp4_row_scales(e8m0)")
     if FUSE_UNPACK if lazy is None else lazy:
-        return PackedWq(codes, bcodes, N, K, fmt)
+        return PackedWq(codes, bcodes, N, K, fmt, wscale)
     assert codes.numel() * codes.element_size() == N * K // 2, "codes must hold N*K/2 bytes"
     wq = torch.empty((N, K), dtype=torch.int8, device=codes.device)
     _lib.call("scmx_unpack_i8", fmt.c_struct(), _lib.ptr(codes), _lib.ptr(bcodes), _lib.ptr(wq), N, K, _lib.stream())
@@ -106,7 +110,8 @@ def _gemm(xq, wq, xscale, wscale, epi, res):
     r = _lib.ptr(res) if epi == 2 else None
     if isinstance(wq, PackedWq):
         _lib.call("scmx_mm_w4a8", wq.fmt.c_struct(), _lib.ptr(xq), _lib.ptr(xscale), _lib.ptr(wq.codes),
-                  _lib.ptr(wq.bcodes), _lib.ptr(wscale), r, _lib.ptr(out), epi, M, N, K, _lib.stream())
+                  _lib.ptr(wq.bcodes), _lib.ptr(wscale if wscale is not None else wq.wscale), r, _lib.ptr(out), epi, M, N,
+                  K, _lib.stream())
     else:
         assert wq.dtype == torch.int8
         _lib.call("scmx_mm_epi", _lib.ptr(xq), _lib.ptr(wq), _lib.ptr(xscale), _lib.ptr(wscale), r, _lib.ptr(out), epi,

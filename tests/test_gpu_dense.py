@@ -307,6 +307,25 @@ def test_config1_m8192_and_m512_equal_row_blocks_of_m2048(S, name, n, k):
         assert torch.equal(big[r0:r0 + 512], S.linear_w4a8(x[r0:r0 + 512].contiguous(), dc, db, dw, n)), (name, r0)
 
 
+@pytest.mark.parametrize("name,m,n,k", [("o_proj", 512, 2048, 2048), ("o_proj", 8192, 2048, 2048), ("down", 512, 2048, 6144),
+                                        ("qkv", 512, 4096, 2048)])
+def test_config1_m512_and_m8192_against_the_oracle(S, name, m, n, k):
+    """BASELINE config 1's other token counts held against the oracle directly (not through another launch): the
+    one-call layer with weights and activations generated as config 0 prescribes, every INT32 accumulator and every
+    bf16 output bit for bit, and the 1e-2 relative Frobenius bound of the float path."""
+    rng = np.random.default_rng(7 * m + n + k)
+    codes, bc, ws, q = layout.quantize(llm_weights(rng, n, k))
+    bits, x = llm_acts(rng, m, k)
+    xq_ref, xs_ref = linear.act_quant(x)
+    acc_ref = linear.int_gemm(xq_ref, q)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    xq, xs = S.act_quant(dev(bits), Mp=m)
+    assert np.array_equal(host(S.mm_i8_i32(xq, S.unpack_i8(dc, db, n, k))), acc_ref)
+    y = host(S.linear_w4a8(dev(bits), dc, db, dw, n))
+    assert np.array_equal(y, linear.epilogue(acc_ref, xs_ref, ws, 1))
+    assert linear.rel_fro(bf16.from_bits(y), linear.float_reference(x, q, ws)) < 1e-2   # the north star's tolerance
+
+
 def test_random_shapes_formats_and_epilogues(S):
     """Fifty seeded random problems (ragged M and N, K of 1 to 8 K steps, every test format, every epilogue) through
     the dense GEMM, and row 0 of each through the GEMV: bit-exact against the oracle."""
