@@ -76,7 +76,8 @@ enum { X_PERM8 = 0, X_HALF = 1, X_PLAIN8 = 2 };
 // `pre` (valid when have_pre): the thread's 16 bytes of the row, x[8 tid .. 8 tid + 7], loaded by the caller BEFORE it
 // requested its first weights.  Loads return in order, so a row read after the weight prefetch could only be used once
 // those weights had arrived; read first, the row is quantized while the weights are still on their way.
-template <int NT, int XMODE>
+// KEEP: rows of up to 8 * NT * KEEP values are read once and stay in registers between the maximum and the rounding.
+template <int NT, int XMODE, int KEEP = 1>
 __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red, u32x4 pre = u32x4{0u, 0u, 0u, 0u},
                            bool have_pre = false) {
     constexpr bool F16 = XMODE == X_HALF;
@@ -130,7 +131,7 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red, u
     }
     // eight values per thread and step, from one 16-byte load (and one of the norm weight for pro 2)
     auto values = [&](int c, float (&v)[8]) {
-        const u32x4 p = have_pre ? pre : *reinterpret_cast<const u32x4*>(xr + 8 * c);   // have_pre: only c == tid is asked for
+        const u32x4 p = (have_pre && c == int(threadIdx.x)) ? pre : *reinterpret_cast<const u32x4*>(xr + 8 * c);
         u32x4 q = u32x4{0u, 0u, 0u, 0u};
         if (a.pro == 2) q = *reinterpret_cast<const u32x4*>(a.nw + 8 * c);
 #pragma unroll
@@ -144,8 +145,8 @@ __device__ float stage_row(const GemvArgs& a, int row, int8_t* sx, float* red, u
             }
         }
     };
-    // Rows of up to 8 * NT * KEEP values are read once and kept in registers between the maximum and the rounding.
-    constexpr int KEEP = 1;   // more would cost the kernel a wave of occupancy (the first weight loads are in flight too)
+    // KEEP = 1 where many waves per CU matter (more costs a wave of occupancy: the first weight loads are in flight too);
+    // 3 for narrow layers with long rows, whose second pass over the row would be a second round trip to memory.
     const bool keep = K <= 8 * NT * KEEP;
     float kept[KEEP][8];
     float amax = 0.0f;
@@ -393,7 +394,7 @@ __device__ __forceinline__ int select_reduce(int (&v)[NV], int lane) {
 // instruction: v_cvt_scalef32_pk_f16_fp4 turns two codes into two half-precision values, sign and block scale
 // included, and v_dot2c_f32_f16 multiplies them with the activations held as half precision.  Every value is an
 // integer below 2^11 and every partial sum one below 2^24, so the FP32 sums are exact and equal the integer ones.
-template <int BATCH, int R, int MODE>
+template <int BATCH, int R, int MODE, int KEEP = 1>
 __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     constexpr int NT = 256;
     constexpr int NV = R * BATCH;
@@ -622,7 +623,9 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
     // ---- driver ---------------------------------------------------------------------------------------------------
     // NB register sets hold the wave's current item and the NB - 1 after it.  All are requested before the
     // activations are staged, so the first weights are already on their way while the workgroup quantizes its input.
-    constexpr int NB = 2;   // a third set costs occupancy and measured slower
+    // a third set costs occupancy and measured slower on wide layers; the long-row variant for narrow layers (KEEP > 1)
+    // has few waves per CU anyway and three items per row, so it requests all of a row's codes at once
+    constexpr int NB = KEEP > 1 ? 3 : 2;
     const auto advance = [&](int& gi, int& cidx) {
         if (++cidx == CI) {
             cidx = 0;
@@ -648,7 +651,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvArgs a) {
 
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-        const float s = stage_row<NT, FP4 ? X_HALF : X_PERM8>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red, xpre, have_pre && b == 0);
+        const float s = stage_row<NT, FP4 ? X_HALF : X_PERM8, KEEP>(a, xrow0 + b, sx + size_t(b) * Kp * XB, red, xpre, have_pre && b == 0);
         for (int c = K * XB / 4 + tid; c < Kp * XB / 4; c += NT) reinterpret_cast<uint32_t*>(sx + size_t(b) * Kp * XB)[c] = 0u;
         if (tid == 0) sxs[b] = s;
     }
@@ -1086,7 +1089,11 @@ static void launch_gemv(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
         kernel<<<grid, block, smem, s>>>(a);
     };
+    // one activation row longer than a pass of the workgroup on a narrow layer: keep the whole row in registers (one trip
+    // to memory for it instead of two; down_proj 2048 x 6144)
+    const bool long_row = BATCH == 1 && R == 1 && a.pro != 0 && a.K > 2048 && a.K <= 6144;
     if (mode == 5) go(gemv_kernel<BATCH, R, 5>);
+    else if (mode == 2 && long_row) go(gemv_kernel<BATCH, R, 2, (BATCH == 1 && R == 1) ? 3 : 1>);
     else if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
     else if (mode == 3) go(gemv_kernel<BATCH, R, 3>);
     else if (mode == 4) go(gemv_kernel<BATCH, R, 4>);
