@@ -50,6 +50,14 @@ typedef struct scmx_format {
 const char* scmx_version(void);
 const char* scmx_last_error(void);
 
+/* Optional set-up for the CURRENT device: looks up the device addresses of the library's two device-resident objects (the
+ * SiLU table of the SwiGLU epilogue and the built-in scratch of scmx_linear_w4a8_static) so that no later call has to.
+ * Those look-ups are runtime calls outside any stream (the first one may load the code object); every entry point
+ * performs them on first use, which is fine in eager code but must not happen while a stream is being captured into a HIP
+ * graph: call scmx_init() once per device (or make one eager call of the entry points you capture) before capturing.
+ * Idempotent, thread-safe, allocates nothing.  No counterpart in the reference (mx.compile needs no such step). */
+int scmx_init(void);
+
 /* Fill `f` with the published SC-MXFP4 format: block 32, magnitudes 2 x E2M1, multipliers 1,2,4,8, 2-bit codes
  * (sc_format.DEFAULT, e2e/sc_format.py:63). */
 void scmx_default_format(scmx_format* f);
@@ -102,7 +110,8 @@ int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* 
  * scratch argument.  No counterpart in the reference.  Limits: M * K <= scmx_linear_w4a8_static_max_elements()
  * (16 Mi) and M <= scmx_linear_w4a8_static_max_rows() (16384); larger shapes return SCMX_ERR_WORKSPACE.  Same results as
  * scmx_linear_w4a8.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
- * or threads) race and must be serialised by the caller; each GPU holds 16.06 MiB for it until the process ends. */
+ * or threads) race and must be serialised by the caller; each GPU holds 16.06 MiB for it until the process ends.
+ * Under graph capture: call scmx_init() (or this entry point once, eagerly) on the device before the capture begins. */
 size_t scmx_linear_w4a8_static_max_elements(void);
 int scmx_linear_w4a8_static_max_rows(void);
 int scmx_linear_w4a8_static(const scmx_format* fmt, const uint16_t* x, const uint32_t* codes, const uint8_t* bcodes,

@@ -21,6 +21,7 @@ _FMT = C.POINTER(CFormat)
 SIGNATURES = {
     "scmx_version": (C.c_char_p, []),
     "scmx_last_error": (C.c_char_p, []),
+    "scmx_init": (_I, []),
     "scmx_default_format": (None, [_FMT]),
     "scmx_mxfp4_format": (None, [_FMT]),
     "scmx_unpack_i8": (_I, [_FMT, _P, _P, _P, _L, _L, _P]),

@@ -877,6 +877,15 @@ static uint8_t* static_scratch_device() {
     return p;
 }
 
+int scmx_init(void) {
+    if (!static_scratch_device()) return SCMX_ERR_LAUNCH;
+    if (!silu_table_device()) {
+        set_error("init: the SiLU table of the SwiGLU epilogue could not be located on the current device");
+        return SCMX_ERR_LAUNCH;
+    }
+    return SCMX_OK;
+}
+
 size_t scmx_linear_w4a8_static_max_elements(void) { return STATIC_XQ_BYTES; }
 int scmx_linear_w4a8_static_max_rows(void) { return STATIC_MAX_ROWS; }
 

@@ -1143,14 +1143,16 @@ static void launch_gemv_rows(const GemvArgs& a, int slots, int dflt, hipStream_t
         if (a.N >= HMFMA_MIN_ROWS && a.K <= 2048 && a.K >= 1536) return launch_gemv_hmfma<BATCH, true>(a, false, s);
         return launch_gemv_hmfma<BATCH, true>(a, true, s);
     }
-    if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 2048 && a.N >= HMFMA_MIN_ROWS)
+    // (both half-precision MFMA kernels read a row's block codes of a piece with one 4-byte load: aligned codes only)
+    const bool bc4 = uintptr_t(a.bcodes) % 4 == 0;
+    if (BATCH > 1 && dflt == 1 && bc4 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 2048 && a.N >= HMFMA_MIN_ROWS)
         return launch_gemv_hmfma<BATCH>(a, false, s);
     // narrow layers with several activation rows: the same kernel with K split over the waves of a workgroup
     // (batch 1 measured no faster this way than with the per-row kernels: qkv 4.70 against 4.40 us, down 7.32 against 6.34)
-    if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 8192 && a.N < HMFMA_MIN_ROWS &&
+    if (BATCH > 1 && dflt == 1 && bc4 && !a.eidx && a.N % 16 == 0 && a.K % 512 == 0 && a.K <= 8192 && a.N < HMFMA_MIN_ROWS &&
         size_t(BATCH) * a.K <= 32768)
         return launch_gemv_hmfma<BATCH>(a, true, s);
-    if (BATCH > 1 && dflt == 1 && !a.eidx && a.N % 4 == 0 && a.K % 512 == 0)
+    if (BATCH > 1 && dflt == 1 && bc4 && !a.eidx && a.N % 4 == 0 && a.K % 512 == 0)
         return launch_gemv_mfma<BATCH>(a, s);
     // more rows per wave = more loads in flight per lane; fewer = more waves for narrow layers
     const long rows = long(a.N) * slots;

@@ -289,3 +289,24 @@ def test_gemv_narrow_layers_split_over_k(G, batch, n, k, pro):
     for b in range(batch):                           # and every row equals its own batch-1 call
         one = host(G.gemv(xin[b], dc, db, None if xsc is None else xsc[b:b + 1], dw, n, 1, **kw))
         assert np.array_equal(one, ref1[b])
+
+
+@pytest.mark.parametrize("n,k", [(36864, 2048), (2048, 2048), (512, 6144)])
+def test_gemv_block_codes_at_an_odd_address(G, n, k):
+    """Block codes that start at an odd byte address (a view into a larger buffer): the wide and the narrow batch
+    kernels read them with 4- and 16-byte loads and are only chosen for aligned codes; every batch gives the bits of
+    the aligned call."""
+    rng = np.random.default_rng(n + k + 1)
+    codes, bc, ws, q = random_packed(rng, n, k)
+    dc, dw = dev(codes), dev(ws)
+    aligned = dev(bc)
+    buf = torch.zeros(bc.size + 64, dtype=torch.uint8, device="cuda")
+    odd = buf[33:33 + bc.size].view(bc.shape)
+    odd.copy_(aligned)
+    assert odd.data_ptr() % 2 == 1
+    for batch in (1, 2, 4, 8):
+        xb, _ = llm_acts(rng, batch, k)
+        dx = dev(xb) if batch > 1 else dev(xb)[0]
+        ya = G.gemv(dx, dc, aligned, None, dw, n, 1, pro=1)
+        yo = G.gemv(dx, dc, odd, None, dw, n, 1, pro=1)
+        assert torch.equal(ya, yo), batch

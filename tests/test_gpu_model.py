@@ -571,3 +571,40 @@ def test_olmoe_decode_continues_the_prefill(tiny_moe, fuse):
     assert rel(rows, full[27:]) < 3e-2, rel(rows, full[27:])
     logits = O.DecodeOlmoe(m).step(ids[:1], m.make_cache(8))
     assert logits.shape == (1, args.vocab_size)
+
+
+@pytest.mark.parametrize("renorm", [False, True])
+def test_olmoe_kernel_router_against_array_op_routing(tiny_moe, renorm):
+    """The router kernel lists a token's experts by falling probability (ties by rising index); the array-op routing it
+    replaced (softmax in float32 -> bf16, `topk(sorted=False)`, optional renormalisation: the reference's
+    e2e/fused_olmoe.py:183-192 with argpartition's order) leaves the order open.  The weighted combine adds the slots
+    one after another in bf16, so the order can move the last bit of a sum and nothing more: the same experts are
+    chosen for every token, with the same scores, and the block outputs of the two routings differ by bf16 rounding."""
+    import types
+    O, args, state, packed = tiny_moe
+    args = O.OlmoeArgs(**{**args.__dict__, "norm_topk_prob": renorm})
+    ids = torch.randint(0, args.vocab_size, (60,), generator=torch.Generator().manual_seed(21)).cuda()
+    m = O.FusedOlmoe(args, state, packed, tile=64)
+    m.record = []
+    h_kernel = m.hidden(ids)
+    kernel_routing = [(i.clone(), s.clone()) for i, s in m.record]
+
+    def array_route(self, nw, xn, M):
+        logits = xn[:M] @ nw["mlp.gate"].T
+        p = torch.softmax(logits.float(), -1).to(torch.bfloat16)
+        scores, inds = torch.topk(p, self.args.num_experts_per_tok, dim=-1, sorted=False)
+        if self.args.norm_topk_prob:
+            scores = scores / scores.sum(-1, keepdim=True)
+        return inds.to(torch.int32), scores
+
+    m2 = O.FusedOlmoe(args, state, packed, tile=64)
+    m2.route = types.MethodType(array_route, m2)
+    m2.record = []
+    h_array = m2.hidden(ids)
+    # layer 0 sees identical inputs: same expert sets, same score per chosen expert
+    (ik, sk), (ia, sa) = kernel_routing[0], m2.record[0]
+    order_k, order_a = ik.long().argsort(-1), ia.long().argsort(-1)
+    assert torch.equal(ik.long().gather(-1, order_k), ia.long().gather(-1, order_a))
+    dk, da = sk.float().gather(-1, order_k), sa.float().gather(-1, order_a)
+    assert float((dk - da).abs().max()) <= 2.0 ** -7 * float(da.abs().max())          # one bf16 step at most
+    assert rel(h_kernel, h_array) < 1e-2, rel(h_kernel, h_array)

@@ -43,12 +43,14 @@ def test_static_scratch_entry_point_equals_the_workspace_one():
                         rp, out_a.data_ptr(), epi, m, n, k, wsp.data_ptr(), need, sp)
         assert rc == 0, msg
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        assert lib.scmx_init() == 0          # address look-ups done: nothing below may change the device's free memory
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         rc, msg = _call(lib, "scmx_linear_w4a8_static", C.byref(fmt), dx.data_ptr(), dc.data_ptr(), db.data_ptr(),
                         dw.data_ptr(), rp, out_b.data_ptr(), epi, m, n, k, sp)
         assert rc == 0, msg
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        # torch's counter sees only torch's allocator; the driver's free-memory figure sees a hipMalloc by anyone
+        assert torch.cuda.memory_allocated() == before and torch.cuda.mem_get_info()[0] == free_before
         assert torch.equal(out_a, out_b), (m, n, k, epi)
         # and both are the oracle's layer
         xq, xs = linear.act_quant(x)
@@ -69,3 +71,43 @@ def test_static_scratch_limits_are_refused():
         assert rc == -4 and "beyond the built-in scratch" in msg
     rc, msg = _call(lib, "scmx_linear_w4a8_static", C.byref(fmt), p, p, p, p, None, p, 1, -1, 128, 128, sp)
     assert rc == -1
+
+
+def test_static_entry_point_inside_a_captured_graph():
+    """The use the entry point is meant for: after scmx_init() on the device, the call is captured into a HIP graph and
+    replayed with changed inputs; every replay equals the eager workspace entry point."""
+    from mxfp4_int8_m5_amd import _lib, sc_format
+    lib = _lib.load()
+    fmt = sc_format.DEFAULT.c_struct()
+    assert lib.scmx_init() == 0
+    rng = np.random.default_rng(78)
+    m, n, k = 192, 512, 1024
+    codes, bc, ws, q = random_packed(rng, n, k)
+    dc, db, dw = dev(codes), dev(bc), dev(ws)
+    x = torch.zeros((m, k), dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((m, n // 2), dtype=torch.bfloat16, device="cuda")       # SwiGLU: the epilogue that reads the table
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        sp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc, msg = _call(lib, "scmx_linear_w4a8_static", C.byref(fmt), x.data_ptr(), dc.data_ptr(), db.data_ptr(),
+                        dw.data_ptr(), None, y.data_ptr(), 3, m, n, k, sp)
+        assert rc == 0, msg
+    torch.cuda.current_stream().wait_stream(side)
+    need = lib.scmx_linear_w4a8_workspace(m, k)
+    wsp = torch.empty(need, dtype=torch.uint8, device="cuda")
+    want = torch.zeros_like(y)
+    sp0 = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for seed in (1, 2, 3):
+        bits, xf = llm_acts(np.random.default_rng(seed), m, k)
+        x.copy_(dev(bits))
+        graph.replay()
+        rc, msg = _call(lib, "scmx_linear_w4a8", C.byref(fmt), x.data_ptr(), dc.data_ptr(), db.data_ptr(), dw.data_ptr(),
+                        None, want.data_ptr(), 3, m, n, k, wsp.data_ptr(), need, sp0)
+        assert rc == 0, msg
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), seed
+        xq, xs = linear.act_quant(xf)
+        with np.errstate(all="ignore"):
+            assert np.array_equal(host(y), linear.epilogue(linear.int_gemm(xq, q), xs, ws, 3)), seed
