@@ -726,11 +726,14 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     // the widest tile only where its tiles fill whole rounds of the CUs (a last round that is mostly empty costs
     // more than the narrower tile's extra LDS traffic: 384 tiles would take 2 rounds of double-size work)
     const long t256 = tiles(256, 256);
-    if (t256 >= cus && t256 * 100 >= ((t256 + cus - 1) / cus) * cus * 88)
+    // ... and one round of them on at least 70 % of the CUs beats the round and a half that the same problem takes as
+    // 256x128 tiles (gate_up at M = 1024: 192 tiles in 33.7 us against 384 in 36.3)
+    const long t256x128 = tiles(256, 128);
+    if ((t256 >= cus && t256 * 100 >= ((t256 + cus - 1) / cus) * cus * 88) ||
+        (t256 < cus && t256 * 100 >= cus * 70 && t256x128 > cus))
         return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
     // ... and one round of 256x128 tiles on at least 70 % of the CUs beats the round and a bit that the same problem takes
     // as 128x128 tiles (gate_up at M = 512: 192 tiles in 19.5 us against 384 in 25.2)
-    const long t256x128 = tiles(256, 128);
     if (t256x128 >= cus || (t256x128 * 100 >= cus * 70 && tiles(128, 128) > cus))
         return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
     if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);

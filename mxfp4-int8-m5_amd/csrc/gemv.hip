@@ -1092,7 +1092,8 @@ static void launch_gemv(const GemvArgs& a, int slots, int dflt, hipStream_t s) {
     // one activation row longer than a pass of the workgroup on a narrow layer: keep the whole row in registers (one trip
     // to memory for it instead of two; down_proj 2048 x 6144)
     const bool long_row = BATCH == 1 && R == 1 && a.pro != 0 && a.K > 2048 && a.K <= 6144;
-    if (mode == 5) go(gemv_kernel<BATCH, R, 5>);
+    if (mode == 5 && long_row) go(gemv_kernel<BATCH, R, 5, (BATCH == 1 && R == 1) ? 3 : 1>);
+    else if (mode == 5) go(gemv_kernel<BATCH, R, 5>);
     else if (mode == 2 && long_row) go(gemv_kernel<BATCH, R, 2, (BATCH == 1 && R == 1) ? 3 : 1>);
     else if (mode == 2) go(gemv_kernel<BATCH, R, 2>);
     else if (mode == 3) go(gemv_kernel<BATCH, R, 3>);

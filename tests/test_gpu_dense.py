@@ -267,7 +267,7 @@ def test_linear_layer_replays_in_a_hip_graph(S):
 
 
 @pytest.mark.parametrize("m,n,k,fmt_i", [(4000, 4096, 256, 0), (4096, 4100, 128, 0), (4096, 4096, 128, 2), (4090, 4096, 384, 1),
-                                          (4096, 4096, 128, 5)])
+                                          (4096, 4096, 128, 5), (760, 16384, 128, 0)])   # the last: 192 tiles, one round
 def test_widest_tile_configuration(S, m, n, k, fmt_i):
     """Problems with at least 256 tiles of 256 x 256 run the widest configuration (wave tiles of 128 x 64, K steps of
     64): ragged last row and column tiles, the published and a generic format, INT32 and all scaling epilogues,
