@@ -90,6 +90,17 @@ int main() {
         ++failures;
     }
 
+    scmx_format mx;
+    scmx_mxfp4_format(&mx);
+    if (mx.block != 32 || mx.bc_bits != 8 || mx.n_mult != 0 || mx.code_mag[7] != 12 || mx.mult[0] != 0) {
+        printf("FAIL MXFP4 in-place format\n");
+        ++failures;
+    }
+    expect(scmx_unpack_i8(&mx, codes, bc, oq, 8, 128, nullptr), SCMX_ERR_FORMAT, "unpack_i8 of the in-place MXFP4 form");
+    expect(scmx_mm_w4a8(&mx, xq, nullptr, codes, bc, nullptr, nullptr, out, 0, 4, 8, 128, nullptr), SCMX_ERR_ARG,
+           "mm_w4a8 in-place MXFP4 without row scales");
+    expect(scmx_mxfp4_to_sc(bc, nullptr, nullptr, oi[0], 8, 128, nullptr), SCMX_ERR_ARG, "mxfp4_to_sc null wscale");
+
     // ---- refused arguments --------------------------------------------------------------------------------------------
     expect(scmx_unpack_i8(nullptr, codes, bc, oq, 8, 128, nullptr), SCMX_ERR_ARG, "unpack_i8 null format");
     expect(scmx_unpack_i8(&fmt, nullptr, bc, oq, 8, 128, nullptr), SCMX_ERR_ARG, "unpack_i8 null codes");

@@ -86,6 +86,32 @@ def test_argument_errors_return_before_any_launch(pkg):
     assert lib.scmx_mm_w4a8(C.byref(fmt), p, p, p, p, p, None, p, 1, 0, 8, 128, None) == 0            # M = 0: nothing to do
 
 
+def test_mxfp4_in_place_descriptor(pkg):
+    """The descriptor of a standard MXFP4 tensor read in place: block 32, one byte per block, no multiplier table; the
+    Python Format and the C filler agree; entry points that cannot decode it without row scales say so before any launch."""
+    lib = pkg._lib.load()
+    F = pkg.sc_format
+    c = pkg._lib.CFormat()
+    lib.scmx_mxfp4_format(C.byref(c))
+    p = F.MXFP4.c_struct()
+    assert (c.block, c.bc_bits, c.n_mult) == (32, 8, 0) == (p.block, p.bc_bits, p.n_mult)
+    assert list(c.code_mag) == list(p.code_mag) == [0, 1, 2, 3, 4, 6, 8, 12] and not any(c.mult) and not any(p.mult)
+    assert F.MXFP4.e8m0 and not F.DEFAULT.e8m0 and F.MXFP4.bits_per_weight(2048) == pytest.approx(4.25 + 32 / 2048)
+    buf = (C.c_char * 4096)()
+    q = C.addressof(buf) // 256 * 256 + 256
+    assert lib.scmx_unpack_i8(C.byref(c), q, q, q, 4, 128, None) == -2 and b"E8M0" in lib.scmx_last_error()
+    assert lib.scmx_mm_w4a8(C.byref(c), q, None, q, q, None, None, q, 0, 4, 8, 128, None) == -1      # INT32 out still needs wscale
+    assert b"wscale" in lib.scmx_last_error()
+    bad = pkg._lib.CFormat()
+    C.memmove(C.byref(bad), C.byref(c), C.sizeof(bad))
+    bad.code_mag[7] = 10                                                                              # not the E2M1 codebook
+    assert lib.scmx_mm_w4a8(C.byref(bad), q, q, q, q, q, None, q, 1, 4, 8, 128, None) == -2
+    with pytest.raises(AssertionError):
+        F.Format(block=16, mult=(), bc_bits=8)
+    with pytest.raises(ValueError):
+        pkg.sc_kernels.unpack_i8(None, None, 4, 128, fmt=F.MXFP4)                                     # no row scales given
+
+
 def test_cpu_tensors_and_missing_library_fail_loudly(pkg, monkeypatch):
     x = torch.zeros((4, 128), dtype=torch.bfloat16)
     with pytest.raises(ValueError):
