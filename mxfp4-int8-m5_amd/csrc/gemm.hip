@@ -50,10 +50,14 @@ enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3,
 // PK (B_PACKED_DEFAULT / B_PACKED_B16, K steps of 128): the weights stay packed in LDS -- 64 bytes of codes per row and
 // K step plus the step's block-code bytes -- and every wave decodes its own fragments after reading them.  Half the
 // weight bytes through LDS in both directions, paid with one decode per wave row that shares the fragment.
-template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false>
-__global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs a) {
+// KG > 1 (small problems: fewer tiles than CUs): KG groups of WGM x WGN waves share the tile, each multiplies its own
+// K / KG of the reduction out of LDS stages of its own, and the INT32 partial sums meet in LDS before the epilogue (exact:
+// integer addition is associative).  A CU then runs KG times the waves on the same tile count.
+template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false,
+          int KG = 1>
+__global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const GemmArgs a) {
     constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
-    constexpr int NT = WGM * WGN * 64;
+    constexpr int NT = WGM * WGN * 64;   // threads of one K group
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int MI = WTM / 32, NI = WTN / 32;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && (BK == 64 || BK == 128), "tile must be whole 32x32x32 MFMAs");
@@ -78,7 +82,15 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // The epilogue reuses the buffer for one [WTM x (row bytes + 16)] output tile per wave; when the bf16 tiles
     // need more than the stages and still fit the CU, the buffer is sized for them.
     constexpr int EPI_BYTES = WGM * WGN * WTM * (WTN * 2 + 16);
-    constexpr int SMEM_BYTES = (EPI_BYTES > NSTAGE * STAGE && EPI_BYTES <= 150 * 1024) ? EPI_BYTES : NSTAGE * STAGE;
+    static_assert(KG == 1 || (!PK && !SKIP), "K groups: staged dense tiles");
+    constexpr int GROUP_BYTES = NSTAGE * STAGE;
+    // after the K loop: group 0's output tiles (the widest epilogue's) from 0, then the other groups' partial sums
+    constexpr int PART_BYTES = NT * MI * NI * 64;
+    constexpr int PART_BASE = WGM * WGN * WTM * (WTN * 4 + 16);
+    constexpr int KG_BYTES = PART_BASE + (KG - 1) * PART_BYTES > KG * GROUP_BYTES ? PART_BASE + (KG - 1) * PART_BYTES : KG * GROUP_BYTES;
+    static_assert(KG == 1 || KG_BYTES <= 160 * 1024, "stages and partial sums fit the CU's LDS");
+    constexpr int SMEM_BYTES =
+        KG > 1 ? KG_BYTES : (EPI_BYTES > NSTAGE * STAGE && EPI_BYTES <= 150 * 1024) ? EPI_BYTES : NSTAGE * STAGE;
     __shared__ __attribute__((aligned(16))) int8_t smem[SMEM_BYTES];
     // scales of the tile's rows and columns, fetched before the K loop so that the epilogue does not start with a
     // round trip to memory
@@ -87,7 +99,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // packed weight rows (64 bytes, 4 chunks): 4 rows per sweep of the banks, chunk c of row r at c ^ ((r / 4) % 4)
     auto swzp = [](int row, int chunk) { return row * (BK / 2) + ((chunk ^ ((row >> 2) & 3)) << 4); };
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = KG == 1 ? 0 : __builtin_amdgcn_readfirstlane(int(threadIdx.x) / NT);   // K group (wave-uniform)
+    const int tid = KG == 1 ? int(threadIdx.x) : int(threadIdx.x) % NT, lane = tid & 63, wave = tid >> 6;
+    int8_t* const sm = smem + kg * GROUP_BYTES;   // this group's stages
     const int wm = SKIP ? wave / WGN : wave % WGM, wn = SKIP ? wave % WGN : wave / WGM;
 
     // ---- which tile ------------------------------------------------------------------------------------------
@@ -124,6 +138,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         row_end = a.M;
     }
     const int K = a.K;
+    const int KL = K / KG;         // length of this group's part of the reduction
+    const int kbase = kg * KL;     // and its first k (a multiple of 128)
     // 32-row blocks of this wave's tile that hold rows of the segment (wave-uniform)
     const int mi_active =
         SKIP ? __builtin_amdgcn_readfirstlane(min(MI, max(0, (row_end - (m0 + wm * WTM) + 31) / 32))) : MI;
@@ -159,7 +175,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         if (m0 + row < row_end) a_live |= 1u << j;
         int gr = min(m0 + row, row_end - 1);   // rows past the segment re-read its last row: one cache line, not a row each
         if (a.gather) gr = a.gather[gr];
-        a_src[j] = int(uint32_t(gr) * uint32_t(K) + kc * 16);
+        a_src[j] = int(uint32_t(gr) * uint32_t(K) + kc * 16 + kbase);
         a_dst[j] = swz(row, kc);
     }
     int b_src[B_PER], b_bc[B_PER], b_dst[B_PER], b_dst2[B_PER], b_k[B_PER];
@@ -170,7 +186,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         if (BMODE == B_INT8) {
             const int row = c / CPR, kc = c % CPR;
             const int gn = min(n0 + row, a.N - 1);
-            b_src[j] = gn * K + kc * 16;
+            b_src[j] = gn * K + kc * 16 + kbase;
             b_dst[j] = BM * BK + swz(row, kc);
             b_dst2[j] = 0;
             b_bc[j] = 0;
@@ -179,13 +195,14 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             constexpr int RUNS = BK / (8 * WPC);   // runs per tile row
             const int row = c / RUNS, kb = c % RUNS;
             const int gn = min(n0 + row, a.N - 1);
-            b_src[j] = gn * (K / 2) + kb * 4 * WPC;
+            b_src[j] = gn * (K / 2) + kb * 4 * WPC + kbase / 2;
             // the block-code byte of the run: 4 blocks per byte, i.e. 128 weights (one byte per K step at most) or 64
             // (two 4-bit codes per byte: 32)
-            b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16    ? (kb * 8 * WPC) >> 6
-                                             : BMODE == B_PACKED_B16M ? (kb * 8 * WPC) >> 5
-                                             : BMODE == B_PACKED_E8M0 ? (kb * 8 * WPC) >> 5
-                                                                      : 0);
+            b_bc[j] = gn * a.bc_row_bytes + (BMODE == B_PACKED_B16      ? (kbase + kb * 8 * WPC) >> 6
+                                             : BMODE == B_PACKED_B16M   ? (kbase + kb * 8 * WPC) >> 5
+                                             : BMODE == B_PACKED_E8M0   ? (kbase + kb * 8 * WPC) >> 5
+                                             : BMODE == B_PACKED_DEFAULT ? kbase >> 7
+                                                                        : 0);
             if (BMODE == B_PACKED_E8M0) b_rmin[j] = e8m0_row_min(a.wscale[erow + gn]);
             if (PK) {   // the run's 16 code bytes as they are
                 b_dst[j] = BM * BK + swzp(row, kb);
@@ -250,7 +267,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             }
     };
     auto load_global = [&](Staged& r, int k0) {
-        k0 = min(k0, K - BK);
+        k0 = min(k0, KL - BK);
 #pragma unroll
         for (int q = 0; q < NKK; ++q) load_slice(r, k0, q);
     };
@@ -259,6 +276,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // step being multiplied: slice q writes the activation chunks j with j % NKK == q and decodes the weight code
     // words w with w * NKK / 4 == q; the last slice writes the decoded weights.
     auto stage_slice = [&](const Staged& r, int8_t* st, int k0, int q, uint32_t (&o)[B_PER][8]) {
+        k0 += kbase;   // block indices below count from the row's first weight
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
             if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS) && (!SKIP || ((a_live >> j) & 1u)))
@@ -304,10 +322,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
             }
     };
     auto store_lds = [&](const Staged& r, int stage, int k0) {
-        k0 = min(k0, K - BK);
+        k0 = min(k0, KL - BK);
         uint32_t o[B_PER][8];
 #pragma unroll
-        for (int q = 0; q < NKK; ++q) stage_slice(r, smem + stage * STAGE, k0, q, o);
+        for (int q = 0; q < NKK; ++q) stage_slice(r, sm + stage * STAGE, k0, q, o);
     };
 
     v16i acc[MI][NI];
@@ -328,7 +346,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     const int a_frag = (wm * WTM + lr) * BK;
     const int b_frag = BM * BK + (wn * WTN + lr) * BK;
 
-    const int KT = K / BK;
+    const int KT = KL / BK;
     // Pipeline.  Iteration kt: barrier; multiply step kt out of its LDS stage while the register set holding step
     // kt+2 is decoded and written into its stage, one slice per 32-wide k slice of MFMAs; then reissue that set's
     // global loads for step kt+4.  A stage is rewritten two barriers after its last read and readable one barrier
@@ -482,7 +500,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         decode_pair(pw[0], bcc, 0, 0, px[0]);
     } else {
 #pragma unroll
-        for (int q = 0; q < AHEAD; ++q) load_frags(smem, q, fa[q], fb[q]);
+        for (int q = 0; q < AHEAD; ++q) load_frags(sm, q, fa[q], fb[q]);
     }
     auto iteration_staged = [&](auto step_tag, Staged& r, int kt) {
         constexpr int rd = decltype(step_tag)::value;        // kt % 3: stage of step kt
@@ -490,11 +508,11 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
         constexpr int nx = (rd + 1) % NSTAGE;                // stage of step kt + 1
         constexpr int ph = (NKK * rd) % FD;                  // fragment buffer of slice 0 of this step (FD divides 6 * NKK)
         __syncthreads();
-        const int8_t* src = smem + rd * STAGE;
-        const int8_t* nxt = smem + nx * STAGE;
-        int8_t* dst = smem + wr * STAGE;
-        const int k2 = min((kt + 2) * BK, K - BK);      // past the end: rewrites a stage nobody reads again
-        const int k4 = min((kt + 4) * BK, K - BK);
+        const int8_t* src = sm + rd * STAGE;
+        const int8_t* nxt = sm + nx * STAGE;
+        int8_t* dst = sm + wr * STAGE;
+        const int k2 = min((kt + 2) * BK, KL - BK);      // past the end: rewrites a stage nobody reads again
+        const int k4 = min((kt + 4) * BK, KL - BK);
         uint32_t o[B_PER][8];
 #pragma unroll
         for (int kk = 0; kk < NKK; ++kk) {
@@ -555,6 +573,29 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
     // stores are 16 bytes per lane over whole contiguous row segments.
     const int N = a.N;
     __syncthreads();   // every wave is done reading the staging buffers
+    if constexpr (KG > 1) {   // the groups' partial sums meet in group 0 (register r of thread t at word r * NT + t)
+        if (kg > 0) {
+            int32_t* part = reinterpret_cast<int32_t*>(smem + PART_BASE + (kg - 1) * PART_BYTES);
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) part[((i * NI + j) * 16 + r) * NT + tid] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kg > 0) return;
+#pragma unroll
+        for (int g = 1; g < KG; ++g) {
+            const int32_t* other = reinterpret_cast<const int32_t*>(smem + PART_BASE + (g - 1) * PART_BYTES);
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] += other[((i * NI + j) * 16 + r) * NT + tid];
+        }
+    }
     auto epilogue = [&](auto epi_tag) {
     constexpr int epi = decltype(epi_tag)::value;
     constexpr int esize = epi == SCMX_EPI_I32 ? 4 : 2;
@@ -682,13 +723,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, OCC) void gemm_kernel(const GemmArgs
 
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false>
+template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false, int KG = 1>
 static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStream_t s) {
     GemmArgs a = a_in;
     if (a.epi == SCMX_EPI_SWIGLU) a.silu = silu_table_device();
     const int num_n = (a.N + BN - 1) / BN;
     if (a.tstart) row_tiles = (row_tiles + 7) & ~7;   // grouped: whole chunks of 8 row-tile slots (spare slots exit at once)
-    const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * 64);
+    const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * KG * 64);
     if constexpr (PK) {   // callers choose this tile for the two FP4-conversion formats only
         if (bmode == B_PACKED_DEFAULT)
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
@@ -696,17 +737,17 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
     } else {
         if (bmode == B_INT8)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_DEFAULT)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16M)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_E8M0)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
         else
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
     }
 }
 
@@ -739,6 +780,10 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
     if (tiles(256, 64) >= cus) return launch_tile<256, 64, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
     if (tiles(128, 64) >= cus) return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
+    // no more 64x64 tiles than CUs: two K groups per tile put eight waves on a CU instead of four (down at M = 512: 18.1
+    // -> 15.3 us, at M = 131 17.6 -> 14.4; three and four groups were not faster, nor two on 128x128 tiles)
+    if (tiles(64, 64) <= cus && a.K % 256 == 0)
+        return launch_tile<64, 64, 128, 2, 2, 1, 2, false, false, 2>(a, bmode, (a.M + 63) / 64, s);
     return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
 }
 

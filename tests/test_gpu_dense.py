@@ -326,6 +326,35 @@ def test_config1_m512_and_m8192_against_the_oracle(S, name, m, n, k):
     assert linear.rel_fro(bf16.from_bits(y), linear.float_reference(x, q, ws)) < 1e-2   # the north star's tolerance
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 2048, 6144), (131, 2048, 2048), (100, 520, 256), (3, 8, 512), (200, 1000, 1280),
+                                   (64, 16384, 768)])
+@pytest.mark.parametrize("fmt_i", [0, 1, 2, 5])
+def test_few_tiles_two_k_groups(S, m, n, k, fmt_i):
+    """Problems with no more 64x64 tiles than CUs (K a multiple of 256) run two K groups per tile whose INT32 partial
+    sums meet in LDS: INT32 output and every epilogue against the oracle, from one K step per group to 24, in four
+    formats (one per decode path of the kernel), from INT8 and from packed weights."""
+    fmt = FORMATS[fmt_i]
+    rng = np.random.default_rng(m + n + k + fmt_i)
+    codes, bc, _, q = random_packed(rng, n, k, fmt)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    xq[0] = 127
+    xs = (np.abs(rng.standard_normal(m)) * 1e-3).astype(F32)
+    ws = (np.abs(rng.standard_normal(n)) * 1e-4).astype(F32)
+    res = bf16.to_bits(rng.standard_normal((m, n)).astype(F32))
+    acc = linear.int_gemm(xq, q)
+    S.set_format(product_format(fmt))
+    try:
+        for lazy in (False, True):
+            wq = S.unpack_i8(dev(codes), dev(bc), n, k, lazy=lazy)
+            assert np.array_equal(host(S.mm_i8_i32(dev(xq), wq)), acc)
+            assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 1)), linear.epilogue(acc, xs, ws, 1))
+            assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 2, res=dev(res))),
+                                  linear.epilogue(acc, xs, ws, 2, res))
+            assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 3)), linear.epilogue(acc, xs, ws, 3))
+    finally:
+        S.set_format(product_format(layout.DEFAULT))
+
+
 def test_random_shapes_formats_and_epilogues(S):
     """Fifty seeded random problems (ragged M and N, K of 1 to 8 K steps, every test format, every epilogue) through
     the dense GEMM, and row 0 of each through the GEMV: bit-exact against the oracle."""
