@@ -502,8 +502,9 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
 #pragma unroll
         for (int q = 0; q < AHEAD; ++q) load_frags(sm, q, fa[q], fb[q]);
     }
-    auto iteration_staged = [&](auto step_tag, Staged& r, int kt) {
+    auto iteration_staged = [&](auto step_tag, auto stage_tag, Staged& r, int kt) __attribute__((always_inline)) {
         constexpr int rd = decltype(step_tag)::value;        // kt % 3: stage of step kt
+        constexpr bool ST = decltype(stage_tag)::value;      // false in the last two steps: nothing left to stage
         constexpr int wr = (rd + 2) % NSTAGE;                // stage of step kt + 2
         constexpr int nx = (rd + 1) % NSTAGE;                // stage of step kt + 1
         constexpr int ph = (NKK * rd) % FD;                  // fragment buffer of slice 0 of this step (FD divides 6 * NKK)
@@ -528,13 +529,13 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                 for (int j = 0; j < NI; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], fa[(ph + kk) % FD][i], acc[i][j], 0, 0, 0);
             }
-            stage_slice(r, dst, k2, kk, o);
+            if constexpr (ST) stage_slice(r, dst, k2, kk, o);
             if (FD > 2) __builtin_amdgcn_sched_barrier(0);
         }
-        load_global(r, k4);
+        if constexpr (ST) load_global(r, k4);
     };
-    auto iteration = [&](auto step_tag, auto parity_tag, Staged& r, int kt) {
-        if constexpr (PK) iteration_pk(step_tag, parity_tag, r, kt); else iteration_staged(step_tag, r, kt);
+    auto iteration = [&](auto step_tag, auto parity_tag, Staged& r, int kt) __attribute__((always_inline)) {
+        if constexpr (PK) iteration_pk(step_tag, parity_tag, r, kt); else iteration_staged(step_tag, std::true_type{}, r, kt);
     };
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
@@ -545,24 +546,81 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     int kt = 0;
     using Even = std::integral_constant<int, 0>;
     using Odd = std::integral_constant<int, 1>;
-    for (; kt + 6 <= KT; kt += 6) {   // kt stays even here: the parity of every copy is fixed
-        iteration(S0{}, Even{}, r0, kt);
-        iteration(S1{}, Odd{}, r1, kt + 1);
-        iteration(S2{}, Even{}, r0, kt + 2);
-        iteration(S0{}, Odd{}, r1, kt + 3);
-        iteration(S1{}, Even{}, r0, kt + 4);
-        iteration(S2{}, Odd{}, r1, kt + 5);
-    }
-    if (kt < KT) {
-        iteration(S0{}, Even{}, r0, kt);
-        if (kt + 1 < KT) {
+    if constexpr (PK) {
+        for (; kt + 6 <= KT; kt += 6) {   // kt stays even here: the parity of every copy is fixed
+            iteration(S0{}, Even{}, r0, kt);
             iteration(S1{}, Odd{}, r1, kt + 1);
-            if (kt + 2 < KT) {
-                iteration(S2{}, Even{}, r0, kt + 2);
-                if (kt + 3 < KT) {
-                    iteration(S0{}, Odd{}, r1, kt + 3);
-                    if (kt + 4 < KT) iteration(S1{}, Even{}, r0, kt + 4);
+            iteration(S2{}, Even{}, r0, kt + 2);
+            iteration(S0{}, Odd{}, r1, kt + 3);
+            iteration(S1{}, Even{}, r0, kt + 4);
+            iteration(S2{}, Odd{}, r1, kt + 5);
+        }
+        if (kt < KT) {
+            iteration(S0{}, Even{}, r0, kt);
+            if (kt + 1 < KT) {
+                iteration(S1{}, Odd{}, r1, kt + 1);
+                if (kt + 2 < KT) {
+                    iteration(S2{}, Even{}, r0, kt + 2);
+                    if (kt + 3 < KT) {
+                        iteration(S0{}, Odd{}, r1, kt + 3);
+                        if (kt + 4 < KT) iteration(S1{}, Even{}, r0, kt + 4);
+                    }
                 }
+            }
+        }
+    } else {
+        // The last two steps find their stages written and have nothing to stage or load: they run as copies without
+        // that work.  Small wave tiles append them at each exit of the staged steps (one predecessor each); larger
+        // ones, with few registers to spare for the copies that so many joins cost, select them by the stage reached;
+        // the largest (128 accumulators, 256x256) keeps every step alike and stages past the end.
+        constexpr bool INLINE_TAIL = MI * NI <= 2, NO_TAIL = MI * NI > 4;
+        const int KM = NO_TAIL ? KT : max(KT - 2, 0);   // steps that stage step kt + 2
+        auto last_two = [&](auto s_first, auto s_second) __attribute__((always_inline)) {
+            iteration_staged(s_first, std::false_type{}, r0, 0);
+            if (KT >= 2) iteration_staged(s_second, std::false_type{}, r0, 0);
+        };
+        auto tail = [&](auto s_first, auto s_second) __attribute__((always_inline)) {
+            if constexpr (INLINE_TAIL) last_two(s_first, s_second);
+        };
+        for (; kt + 6 <= KM; kt += 6) {
+            iteration(S0{}, Even{}, r0, kt);
+            iteration(S1{}, Odd{}, r1, kt + 1);
+            iteration(S2{}, Even{}, r0, kt + 2);
+            iteration(S0{}, Odd{}, r1, kt + 3);
+            iteration(S1{}, Even{}, r0, kt + 4);
+            iteration(S2{}, Odd{}, r1, kt + 5);
+        }
+        if (kt < KM) {
+            iteration(S0{}, Even{}, r0, kt);
+            if (kt + 1 < KM) {
+                iteration(S1{}, Odd{}, r1, kt + 1);
+                if (kt + 2 < KM) {
+                    iteration(S2{}, Even{}, r0, kt + 2);
+                    if (kt + 3 < KM) {
+                        iteration(S0{}, Odd{}, r1, kt + 3);
+                        if (kt + 4 < KM) {
+                            iteration(S1{}, Even{}, r0, kt + 4);
+                            tail(S2{}, S0{});
+                        } else {
+                            tail(S1{}, S2{});
+                        }
+                    } else {
+                        tail(S0{}, S1{});
+                    }
+                } else {
+                    tail(S2{}, S0{});
+                }
+            } else {
+                tail(S1{}, S2{});
+            }
+        } else {
+            tail(S0{}, S1{});
+        }
+        if constexpr (!INLINE_TAIL && !NO_TAIL) {
+            switch (KM % 3) {
+                case 0: last_two(S0{}, S1{}); break;
+                case 1: last_two(S1{}, S2{}); break;
+                default: last_two(S2{}, S0{}); break;
             }
         }
     }
