@@ -417,6 +417,10 @@ def main():
                     ms_d, ms_d_min = timeit(lambda i: check(lib.scmx_gemv(*argl[i % copies])), reps_d, reps=a.reps, warmup=copies,
                                        warm_s=0.2)
                     us = ms_d * 1e3
+                    # the same call on one weight set over and over: what the layer costs when its weights stay in the
+                    # last-level cache (the protocol of e2e/bench_gemv_qwen35.py:16-18 reports both)
+                    ms_r, _ = timeit(lambda i: check(lib.scmx_gemv(*argl[0])), reps_d, reps=max(3, a.reps // 2), warmup=5,
+                                     warm_s=0.05)
                     # the same launches replayed from a HIP graph: kernel time without the host's per-call launch cost
                     ncap = min(copies, 40)
                     side = torch.cuda.Stream()
@@ -433,6 +437,7 @@ def main():
                     decode[f"{name}_b{batch}{form}"] = {"us": round(us, 2), "us_min": round(ms_d_min * 1e3, 2),
                                                   "gbps": round(bts / us / 1e3, 1),
                                                   "pct_hbm": round(bts / us / 1e3 / PEAK_HBM_GBPS * 100, 1),
+                                                  "us_resident": round(ms_r * 1e3, 2),
                                                   "us_graph": round(us_g, 2), "gbps_graph": round(bts / us_g / 1e3, 1),
                                                   "pct_hbm_graph": round(bts / us_g / 1e3 / PEAK_HBM_GBPS * 100, 1)}
                     del graph
