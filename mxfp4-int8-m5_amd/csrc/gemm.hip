@@ -678,6 +678,8 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
             for (int g = 0; g < 4; ++g)
                 wsv[j][g] = *reinterpret_cast<const f32x4*>(&s_ws[wn * WTN + j * 32 + 8 * g + 4 * half]);
     }
+    auto emit = [&](auto wide_tag) __attribute__((always_inline)) {
+    constexpr bool W = decltype(wide_tag)::value;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
         const int row = i * 32 + lr;
@@ -691,7 +693,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                 const int n = wn0 + col;
                 if (epi == SCMX_EPI_I32) {
                     const v4i v = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    if (wide)
+                    if (W)
                         *reinterpret_cast<v4i*>(wtile + row * rsb + col * 4) = v;
                     else if (m < row_end && n < N)
                         *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(a.out) + size_t(m) * N + n) = v;
@@ -707,7 +709,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                     const uint16_t s0 = swiglu_lut(a.silu, y[0], round_bf16(y[2]));
                     const uint16_t s1 = swiglu_lut(a.silu, y[1], round_bf16(y[3]));
                     const uint32_t o = uint32_t(s0) | (uint32_t(s1) << 16);
-                    if (wide)
+                    if (W)
                         *reinterpret_cast<uint32_t*>(wtile + row * rsb + col) = o;
                     else if (m < row_end && n < N)
                         *reinterpret_cast<uint32_t*>(out + size_t(m) * on + n / 2) = o;
@@ -716,7 +718,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                 u32x2 o;
                 o[0] = uint32_t(f32_to_bf16(y[0])) | (uint32_t(f32_to_bf16(y[1])) << 16);
                 o[1] = uint32_t(f32_to_bf16(y[2])) | (uint32_t(f32_to_bf16(y[3])) << 16);
-                if (wide) {
+                if (W) {
                     *reinterpret_cast<u32x2*>(wtile + row * rsb + col * 2) = o;   // the residual is added on the way out
                 } else if (m < row_end && n < N) {
                     if (epi == SCMX_EPI_RES) {
@@ -733,6 +735,8 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
             }
         }
     }
+    };
+    if (wide) emit(std::true_type{}); else emit(std::false_type{});
     if (!wide) return;
     __builtin_amdgcn_wave_barrier();   // LDS operations of one wave complete in order: the tile is visible to its lanes
 
