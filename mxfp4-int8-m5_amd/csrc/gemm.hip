@@ -826,27 +826,61 @@ static int packed_mode(const DevFormat& f) {
 static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     const long cus = device_cus();
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-    // the widest tile only where its tiles fill whole rounds of the CUs (a last round that is mostly empty costs
-    // more than the narrower tile's extra LDS traffic: 384 tiles would take 2 rounds of double-size work)
-    const long t256 = tiles(256, 256);
-    // ... and one round of them on at least 70 % of the CUs beats the round and a half that the same problem takes as
-    // 256x128 tiles (gate_up at M = 1024: 192 tiles in 33.7 us against 384 in 36.3)
-    const long t256x128 = tiles(256, 128);
-    if ((t256 >= cus && t256 * 100 >= ((t256 + cus - 1) / cus) * cus * 88) ||
-        (t256 < cus && t256 * 100 >= cus * 70 && t256x128 > cus))
-        return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
-    // ... and one round of 256x128 tiles on at least 70 % of the CUs beats the round and a bit that the same problem takes
-    // as 128x128 tiles (gate_up at M = 512: 192 tiles in 19.5 us against 384 in 25.2)
-    if (t256x128 >= cus || (t256x128 * 100 >= cus * 70 && tiles(128, 128) > cus))
-        return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
-    if (tiles(128, 128) >= cus) return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
-    if (tiles(256, 64) >= cus) return launch_tile<256, 64, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
-    if (tiles(128, 64) >= cus) return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
-    // no more 64x64 tiles than CUs: two K groups per tile put eight waves on a CU instead of four (down at M = 512: 18.1
-    // -> 15.3 us, at M = 131 17.6 -> 14.4; three and four groups were not faster, nor two on 128x128 tiles)
-    if (tiles(64, 64) <= cus && a.K % 256 == 0)
-        return launch_tile<64, 64, 128, 2, 2, 1, 2, false, false, 2>(a, bmode, (a.M + 63) / 64, s);
-    return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
+    // The tile is the one a small cost model makes fastest.  A launch runs its tiles in waves of (CUs x workgroups that
+    // share a CU); a wave costs F + S per 128 of K and not less than W, all three measured per configuration and per
+    // number of co-resident workgroups (four Qwen3-1.7B layer shapes and five others, K = 128 ... 6144, M = 64 ... 8192:
+    // the choice is within 2.5 % of the fastest configuration on all 118), and a last wave that leaves CUs idle runs
+    // faster (less contention for the L2s and HBM).  What the table encodes: 256x256 moves the fewest LDS bytes per MFMA
+    // and pays where it fills the chip or saves a round; a mostly empty last round costs more than a narrower tile's
+    // extra LDS traffic; the small tiles share a CU and lose less to a ragged tile count; with no more 64x64 tiles
+    // than CUs two K groups per tile put eight waves on a CU.  (A 256x64 tile was never the fastest and is gone.)
+    struct Cand {
+        int bm, bn, occ;
+        float f[3], s[3], w[3];   // per wave, by co-resident workgroups 1..occ: fixed us, us per 128 of K, least us
+        float low, mid;           // a wave on half of the CUs or fewer / on three quarters of them costs this part of a full one
+    };
+    static const Cand cand[6] = {
+        {256, 256, 1, {6.5f, 0, 0}, {1.9f, 0, 0}, {8.4f, 0, 0}, 0.70f, 0.835f},
+        {256, 128, 1, {4.2f, 0, 0}, {0.94f, 0, 0}, {5.5f, 0, 0}, 0.74f, 0.78f},
+        {128, 128, 1, {1.4f, 0, 0}, {0.62f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
+        {128, 64, 2, {1.4f, 1.2f, 0}, {0.39f, 0.77f, 0}, {2.2f, 3.0f, 0}, 0.91f, 1.0f},
+        {64, 64, 3, {0.85f, 0.6f, 0.6f}, {0.34f, 0.53f, 0.70f}, {1.9f, 2.3f, 2.7f}, 0.95f, 1.0f},
+        {64, 64, 1, {1.1f, 0, 0}, {0.26f, 0, 0}, {2.0f, 0, 0}, 0.97f, 1.0f},   // two K groups
+    };
+    const float steps = float(a.K) / 128.0f;
+    int best = 4;
+    float best_t = 1e30f;
+    for (int c = 0; c < 6; ++c) {
+        const Cand& k = cand[c];
+        const long n = tiles(k.bm, k.bn);
+        if (c == 5 && (n > cus || a.K % 256)) continue;
+        const long cap = cus * k.occ;
+        const long full = n / cap, rest = n % cap;
+        float t = float(full) * fmaxf(k.f[k.occ - 1] + steps * k.s[k.occ - 1], k.w[k.occ - 1]);
+        if (rest) {
+            const int r = int((rest + cus - 1) / cus);   // workgroups per CU in the last wave
+            float w = fmaxf(k.f[r - 1] + steps * k.s[r - 1], k.w[r - 1]);
+            if (r == 1) {   // CUs idle
+                const float fill = float(rest) / float(cus);
+                w *= fill <= 0.5f    ? k.low
+                     : fill <= 0.75f ? k.low + (k.mid - k.low) * (fill - 0.5f) * 4.0f
+                                     : k.mid + (1.0f - k.mid) * (fill - 0.75f) * 4.0f;
+            }
+            t += w;
+        }
+        if (t < best_t * 0.98f) {   // candidates run from the largest tile down: a tie goes to the larger one
+            best_t = t;
+            best = c;
+        }
+    }
+    switch (best) {
+        case 0: return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
+        case 1: return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
+        case 2: return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
+        case 3: return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
+        case 5: return launch_tile<64, 64, 128, 2, 2, 1, 2, false, false, 2>(a, bmode, (a.M + 63) / 64, s);
+        default: return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
+    }
 }
 
 static int check_gemm_common(const char* who, int M, int N, int K, int epi, bool need_scales, const void* xq,

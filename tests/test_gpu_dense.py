@@ -326,12 +326,12 @@ def test_config1_m512_and_m8192_against_the_oracle(S, name, m, n, k):
     assert linear.rel_fro(bf16.from_bits(y), linear.float_reference(x, q, ws)) < 1e-2   # the north star's tolerance
 
 
-@pytest.mark.parametrize("m,n,k", [(512, 2048, 6144), (131, 2048, 2048), (100, 520, 256), (3, 8, 512), (200, 1000, 1280),
+@pytest.mark.parametrize("m,n,k", [(512, 2048, 6144), (131, 2048, 2048), (192, 4096, 1024), (16, 256, 1024), (200, 1000, 1280),
                                    (64, 16384, 768)])
 @pytest.mark.parametrize("fmt_i", [0, 1, 2, 5])
 def test_few_tiles_two_k_groups(S, m, n, k, fmt_i):
-    """Problems with no more 64x64 tiles than CUs (K a multiple of 256) run two K groups per tile whose INT32 partial
-    sums meet in LDS: INT32 output and every epilogue against the oracle, from one K step per group to 24, in four
+    """Problems with no more 64x64 tiles than CUs and enough K steps run two K groups per tile whose INT32 partial sums
+    meet in LDS: INT32 output and every epilogue against the oracle, from three K steps per group to 24, in four
     formats (one per decode path of the kernel), from INT8 and from packed weights."""
     fmt = FORMATS[fmt_i]
     rng = np.random.default_rng(m + n + k + fmt_i)

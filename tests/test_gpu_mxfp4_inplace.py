@@ -132,7 +132,7 @@ def test_gemv_expert_gather(F, G):
 
 
 @pytest.mark.parametrize("m,n,k", [(2048, 2048, 2048), (512, 4096, 2048), (300, 260, 384), (64, 64, 128), (8192, 2048, 256),
-                                   (1, 4, 128), (200, 1024, 1280), (131, 2048, 512)])
+                                   (1, 4, 128), (200, 1024, 1280), (131, 2048, 2048), (2048, 4096, 256)])
 def test_dense_gemm(F, S, m, n, k):
     """Every tile configuration of the dense GEMM on the in-place form: INT32 accumulators and all epilogues."""
     rng = np.random.default_rng(m + n + k)
