@@ -55,12 +55,13 @@ class OlmoeArgs:
 
 
 class FusedOlmoe:
-    def __init__(self, args, params, flat, tile=256, two_pass=False, sort="count", fmt=None, device="cuda"):
+    def __init__(self, args, params, flat, tile=None, two_pass=False, sort="count", fmt=None, device="cuda"):
         """params: Hugging Face names ("model.embed_tokens.weight", "model.norm.weight", "lm_head.weight", per layer
         "model.layers.{i}.input_layernorm.weight", ".post_attention_layernorm.weight", ".self_attn.q_norm.weight",
         ".self_attn.k_norm.weight", ".mlp.gate.weight").  flat: {"layers.{i}.{path}": (codes, bcodes, wscale)} for the
         attention linears and "layers.{i}.experts.{name}.{e}" for the experts (the reference's cache keys).
-        tile: row tile of the grouped GEMM (64, 128 or 256); two_pass: unpack all experts to INT8 first
+        tile: row tile of the grouped GEMM (64, 128 or 256; None: by the rows per expert of each call,
+        sc_moe.row_tile); two_pass: unpack all experts to INT8 first
         (e2e/fused_olmoe.py:133-138); sort: "count" (route_sort kernel) or "argsort" (array ops)."""
         self.args, self.device, self.tile, self.two_pass, self.sort = args, device, tile, two_pass, sort
         self.fmt = fmt if fmt is not None else F.Format()
@@ -134,8 +135,9 @@ class FusedOlmoe:
 
     def _experts(self, xq, xs, inds, scores, h, nn, ex, L, quant=True):
         a = self.args
-        E, F2, D, tm = a.num_experts, 2 * a.intermediate_size, a.hidden_size, self.tile
+        E, F2, D = a.num_experts, 2 * a.intermediate_size, a.hidden_size
         R = L * a.num_experts_per_tok
+        tm = self.tile or sc_moe.row_tile(R, E)
         if self.sort == "count":
             pos, tok, _, off, tstart, maxt = sc_moe.route_sort(inds, E, tm)
         else:   # array ops, as mlx_lm's _gather_sort (e2e/fused_olmoe.py:225-231)

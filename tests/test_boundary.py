@@ -159,6 +159,8 @@ def test_attention_split_policy_and_cache_names(pkg):
     assert (f.block, f.bc_bits, tuple(f.mult)) == (16, 4, tuple(range(1, 11)))
     f = PF.sc_format_of("e2m1/B32/pow2")
     assert (f.block, f.bc_bits, tuple(f.mult)) == (32, 2, (1, 2, 4, 8))
+    # row tile of the grouped GEMM by rows per expert (64 experts: 512 tokens x 8 -> 64 rows each, 1024 -> 128)
+    assert [pkg.sc_moe.row_tile(t * 8, 64) for t in (1, 512, 767, 768, 4096)] == [64, 64, 64, 256, 256]
 
 
 @pytest.mark.skipif(shutil.which(os.environ.get("HIPCC", "hipcc")) is None, reason="needs hipcc to build the instrumented library")

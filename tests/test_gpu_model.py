@@ -537,7 +537,7 @@ def moe_float_model(args, state, packed, ids, routing):
     return norm(h, state["model.norm.weight"])
 
 
-@pytest.mark.parametrize("kw", [dict(tile=64), dict(tile=256, two_pass=True), dict(tile=128, sort="argsort")])
+@pytest.mark.parametrize("kw", [dict(tile=64), dict(tile=256, two_pass=True), dict(tile=128, sort="argsort"), dict()])
 def test_olmoe_prefill_against_float_model(tiny_moe, kw):
     O, args, state, packed = tiny_moe
     ids = torch.randint(0, args.vocab_size, (45,), generator=torch.Generator().manual_seed(11))
