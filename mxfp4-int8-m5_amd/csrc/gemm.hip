@@ -379,6 +379,10 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     store_lds(r0, 0, 0);
     store_lds(r1, 1, BK);
     load_global(r0, 2 * BK);
+    // the two sets' loads stay apart, in the order the K loop issues them: its first copy has two predecessors (this code
+    // and the loop's end) and waits for the fewer outstanding loads of the two -- interleaved here, that wait covered
+    // the younger set as well, in every trip
+    __builtin_amdgcn_sched_barrier(0);
     load_global(r1, 3 * BK);
     // ---- PK: fragments of packed weights ------------------------------------------------------------------------
     // The k positions of a 64-wide pair of MFMA slices are dealt so that a lane's packed codes are one 16-byte read:
