@@ -17,7 +17,8 @@ def gemv(xq, codes, bcodes, xscale, wscale, N, epi, dtype=torch.bfloat16, res=No
          pro=0, nw=None, eps=None, rows=None, vpl=None, shared=None, splitk=None, fmt=None):
     """W4A8 GEMV.  pro=0: xq int8 [K] (or rows) with xscale; pro=1: xq is a bf16 row quantized in the kernel;
     pro=2: RMSNorm(nw, eps) + INT8 in the kernel.  Output EPI 1: [N]; 2: [N] = res + y; 3: [N/2].
-    xq [B, K] with B = 2 ... 8 rows shares one pass over the weights (rows 3, 5, 6, 7 are padded to 4 / 8).
+    xq [B, K] with B = 2 ... 8 rows shares one pass over the weights (3, 5, 6, 7 rows are padded to 4 / 8; more than 8
+    rows take one pass per eight -- from a few dozen rows on the dense GEMM is the faster path).
     MoE (eidx int32 [S]): codes [E, ..], wscale [E, N]; slot j uses expert eidx[j] and input row j if xstride=1;
     shared=e adds one slot for expert e -> [S(+1), N or N/2]."""
     S._check_dtype(dtype)
@@ -30,6 +31,11 @@ def gemv(xq, codes, bcodes, xscale, wscale, N, epi, dtype=torch.bfloat16, res=No
         slots = nslot + (shared is not None)
         eidx = eidx if eidx.dtype == torch.int32 else eidx.view(torch.int32) if eidx.element_size() == 4 else eidx.to(torch.int32)
         out = torch.empty((slots, no), dtype=torch.bfloat16, device=xq.device)
+    elif xq.dim() == 2 and xq.shape[0] > 8:   # more rows than one pass takes: eight at a time
+        cut = lambda t, i: None if t is None else t[i:i + 8]   # noqa: E731
+        return torch.cat([gemv(xq[i:i + 8], codes, bcodes, cut(xscale, i), wscale, N, epi, dtype, cut(res, i), nsg, None,
+                               xstride, pro, nw, eps, rows, vpl, shared, splitk, fmt).reshape(-1, no)
+                          for i in range(0, xq.shape[0], 8)])
     elif xq.dim() == 2 and xq.shape[0] in (3, 5, 6, 7):   # the kernels take 1, 2, 4 or 8 rows: pad with zero rows
         b, bp = xq.shape[0], 4 if xq.shape[0] == 3 else 8
         pad = lambda t: None if t is None else torch.cat([t, t.new_zeros((bp - b,) + tuple(t.shape[1:]))])   # noqa: E731

@@ -108,10 +108,10 @@ def test_gemv_fused_prologues(G, S, pro):
     assert np.array_equal(y0, linear.gemv(rq[0], rs[0], q, ws, 1))
 
 
-@pytest.mark.parametrize("batch", [2, 3, 4, 5, 7, 8])
+@pytest.mark.parametrize("batch", [2, 3, 4, 5, 7, 8, 9, 19])
 def test_gemv_batch_equals_rows(G, batch):
     """B rows against one pass over the weights give the bits of B independent batch-1 GEMVs (3, 5, 6 and 7 rows run
-    padded to 4 / 8 by the Python surface)."""
+    padded to 4 / 8 by the Python surface, more than 8 rows eight at a time)."""
     rng = np.random.default_rng(batch)
     n, k = 1024, 2048
     codes, bc, ws, q = random_packed(rng, n, k)
