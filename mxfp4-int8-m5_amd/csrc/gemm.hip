@@ -506,10 +506,9 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
 #pragma unroll
         for (int q = 0; q < AHEAD; ++q) load_frags(sm, q, fa[q], fb[q]);
     }
-    // The k slices of an iteration are fenced against each other for the scheduler where fragments run more than one
-    // slice ahead, and on the largest wave tile: left alone there, the compiler sinks every LDS write of the step to its
-    // end, in front of the barrier (M = 8192: 442 -> 429 us over the four layers with the fences).
-    constexpr bool FENCE = FD > 2 || MI * NI >= 8;
+    // The k slices of an iteration are fenced against each other for the scheduler: left alone, the compiler sinks every
+    // LDS write of the step to its end, in front of the barrier (M = 8192: 442 -> 429 us over the four layers with the
+    // fences on the 256x256 tile; M = 128 ... 1024 on the small tiles: 2-3 %).
     auto iteration_staged = [&](auto step_tag, auto stage_tag, Staged& r, int kt) __attribute__((always_inline)) {
         constexpr int rd = decltype(step_tag)::value;        // kt % 3: stage of step kt
         constexpr bool ST = decltype(stage_tag)::value;      // false in the last two steps: nothing left to stage
@@ -529,7 +528,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                 load_frags(src, kk + AHEAD, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
             else
                 load_frags(nxt, kk + AHEAD - NKK, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
-            if (FENCE) __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 if (SKIP && i >= mi_active) continue;
@@ -538,7 +537,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], fa[(ph + kk) % FD][i], acc[i][j], 0, 0, 0);
             }
             if constexpr (ST) stage_slice(r, dst, k2, kk, o);
-            if (FENCE) __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (ST) load_global(r, k4);
     };
