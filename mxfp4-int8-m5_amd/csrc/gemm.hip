@@ -751,35 +751,55 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     constexpr int ppr = rowb / 16;                 // 16-byte pieces per tile row (2, 4, 8 or 16)
     constexpr int epp = 16 / esize;                // output elements per piece
     const int ocol0 = epi == SCMX_EPI_SWIGLU ? wn0 / 2 : wn0;
-    for (int p = lane; p < WTM * ppr; p += 64) {
-        const int row = p / ppr, pc = p % ppr;
-        const int m = wm0 + row, c = ocol0 + pc * epp;
-        if (m >= row_end || c >= on) continue;
-        u32x4 v = *reinterpret_cast<const u32x4*>(wtile + row * rsb + pc * 16);
-        int8_t* dst = reinterpret_cast<int8_t*>(a.out) + (size_t(m) * on + c) * esize;
-        if (epi == SCMX_EPI_RES) {
-            const bool full = c + epp <= on;
-            u32x4 rr = u32x4{0u, 0u, 0u, 0u};
-            if (full) {
-                rr = *reinterpret_cast<const u32x4*>(a.res + size_t(m) * on + c);
-            } else {
-                const u32x2 r2 = *reinterpret_cast<const u32x2*>(a.res + size_t(m) * on + c);
-                rr[0] = r2[0];
-                rr[1] = r2[1];
-            }
+    // In batches of eight pieces per lane: all LDS reads (and residual loads) of a batch are in flight before the first
+    // is used, instead of one round trip per piece.
+    constexpr int NP = WTM * ppr / 64, NB = NP < 8 ? NP : 8;
+    static_assert(WTM * ppr % 64 == 0 && NP % NB == 0, "whole batches of pieces per lane");
+#pragma unroll 1
+    for (int p0 = lane; p0 < WTM * ppr; p0 += 64 * NB) {
+        u32x4 v[NB], rr[NB];
+        bool ok[NB], full[NB];
+        int8_t* dst[NB];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float lo = __fadd_rn(__uint_as_float(rr[r] << 16), __uint_as_float(v[r] << 16));
-                const float hi = __fadd_rn(__uint_as_float(rr[r] & 0xFFFF0000u), __uint_as_float(v[r] & 0xFFFF0000u));
-                v[r] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+        for (int i = 0; i < NB; ++i) {
+            const int p = p0 + 64 * i;
+            const int row = p / ppr, pc = p % ppr;
+            const int m = wm0 + row, c = ocol0 + pc * epp;
+            ok[i] = m < row_end && c < on;
+            full[i] = c + epp <= on;
+            dst[i] = reinterpret_cast<int8_t*>(a.out) + (size_t(m) * on + c) * esize;
+            v[i] = *reinterpret_cast<const u32x4*>(wtile + row * rsb + pc * 16);
+            if (epi == SCMX_EPI_RES) {
+                rr[i] = u32x4{0u, 0u, 0u, 0u};
+                if (ok[i]) {
+                    if (full[i]) {
+                        rr[i] = *reinterpret_cast<const u32x4*>(a.res + size_t(m) * on + c);
+                    } else {
+                        const u32x2 r2 = *reinterpret_cast<const u32x2*>(a.res + size_t(m) * on + c);
+                        rr[i][0] = r2[0];
+                        rr[i][1] = r2[1];
+                    }
+                }
             }
         }
-        if (c + epp <= on)
-            // streaming store: the tile is not read again by this kernel, and lines that never sit dirty in the L2
-            // do not have to be written back when the kernel ends
-            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
-        else   // the row ends inside this piece: rows are multiples of 4 elements, so exactly half of it is valid
-            *reinterpret_cast<u32x2*>(dst) = u32x2{v[0], v[1]};
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            if (!ok[i]) continue;
+            if (epi == SCMX_EPI_RES) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float lo = __fadd_rn(__uint_as_float(rr[i][r] << 16), __uint_as_float(v[i][r] << 16));
+                    const float hi = __fadd_rn(__uint_as_float(rr[i][r] & 0xFFFF0000u), __uint_as_float(v[i][r] & 0xFFFF0000u));
+                    v[i][r] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+                }
+            }
+            if (full[i])
+                // streaming store: the tile is not read again by this kernel, and lines that never sit dirty in the L2
+                // do not have to be written back when the kernel ends
+                __builtin_nontemporal_store(v[i], reinterpret_cast<u32x4*>(dst[i]));
+            else   // the row ends inside this piece: rows are multiples of 4 elements, so exactly half of it is valid
+                *reinterpret_cast<u32x2*>(dst[i]) = u32x2{v[i][0], v[i][1]};
+        }
     }
     };
     switch (a.epi) {
