@@ -415,6 +415,8 @@ __global__ __launch_bounds__(RS_CHUNK) void route_place_kernel(const int32_t* __
 }
 
 // ---- MoE: weighted combine of the top-k expert outputs, sequential in bf16 ---------------------------------------
+// W = elements per thread and pass: 8 (16-byte loads) where K and the pointers allow, else 4.
+template <int W>
 __global__ __launch_bounds__(NT) void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ pos,
                                                          const uint16_t* __restrict__ scores, const uint16_t* __restrict__ sscore,
                                                          const uint16_t* __restrict__ res, const uint16_t* __restrict__ w,
@@ -424,16 +426,19 @@ __global__ __launch_bounds__(NT) void moe_combine_kernel(const uint16_t* __restr
     uint16_t* hrow_s = srow;
     uint16_t* nrow_s = srow + K;
     float* red = reinterpret_cast<float*>(srow + 2 * K);
+    using vec = typename std::conditional<W == 8, u32x4, u32x2>::type;
     const int row = blockIdx.x;
     const int nsc = sscore ? topk - 1 : topk;
-    for (int c = threadIdx.x; c < K / 4; c += NT) {
-        const u32x2 r2 = *reinterpret_cast<const u32x2*>(res + size_t(row) * K + 4 * c);
-        u32x2 o = r2;
+    for (int c = threadIdx.x; c < K / W; c += NT) {
+        const vec r2 = *reinterpret_cast<const vec*>(res + size_t(row) * K + W * c);
+        vec o = r2;
         if (row < M) {
-            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float acc[W];
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc[i] = 0.0f;
             // the slots' rows are requested eight at a time, then added in slot order
             for (int j0 = 0; j0 < topk; j0 += 8) {
-                u32x2 y2[8];
+                vec y2[8];
                 float sc[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
@@ -441,29 +446,28 @@ __global__ __launch_bounds__(NT) void moe_combine_kernel(const uint16_t* __restr
                     if (j < topk) {
                         const int p = pos[row * topk + j];
                         sc[u] = bf16_to_f32((sscore && j == topk - 1) ? sscore[row] : scores[row * nsc + j]);
-                        y2[u] = *reinterpret_cast<const u32x2*>(y + size_t(p) * K + 4 * c);
+                        y2[u] = *reinterpret_cast<const vec*>(y + size_t(p) * K + W * c);
                     }
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     if (j0 + u >= topk) break;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
+                    for (int i = 0; i < W; ++i) {
                         const float yv = __uint_as_float(i & 1 ? (y2[u][i >> 1] & 0xFFFF0000u) : (y2[u][i >> 1] << 16));
                         acc[i] = round_bf16(__fadd_rn(round_bf16(__fmul_rn(yv, sc[u])), acc[i]));
                     }
                 }
             }
-            uint16_t hb[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float rv = __uint_as_float(i & 1 ? (r2[i >> 1] & 0xFFFF0000u) : (r2[i >> 1] << 16));
-                hb[i] = f32_to_bf16(__fadd_rn(rv, acc[i]));
+            for (int i = 0; i < W / 2; ++i) {
+                const float lo = __fadd_rn(__uint_as_float(r2[i] << 16), acc[2 * i]);
+                const float hi = __fadd_rn(__uint_as_float(r2[i] & 0xFFFF0000u), acc[2 * i + 1]);
+                o[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
             }
-            o = u32x2{uint32_t(hb[0]) | (uint32_t(hb[1]) << 16), uint32_t(hb[2]) | (uint32_t(hb[3]) << 16)};
         }
-        *reinterpret_cast<u32x2*>(hrow_s + 4 * c) = o;
-        *reinterpret_cast<u32x2*>(h + size_t(row) * K + 4 * c) = o;
+        *reinterpret_cast<vec*>(hrow_s + W * c) = o;
+        *reinterpret_cast<vec*>(h + size_t(row) * K + W * c) = o;
     }
     __syncthreads();
     if (!xq) return;
@@ -713,8 +717,12 @@ int scmx_moe_combine(const uint16_t* y, const int32_t* pos, const uint16_t* scor
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
-    moe_combine_kernel<<<dim3(Mp), dim3(NT), size_t(K) * 4 + 72 * 4, (hipStream_t)stream>>>(y, pos, scores, sscore, res, w,
-                                                                                             eps, h, xq, xs, M, K, topk);
+    if (K % 8 == 0 && (uintptr_t(y) | uintptr_t(res) | uintptr_t(h)) % 16 == 0)
+        moe_combine_kernel<8><<<dim3(Mp), dim3(NT), size_t(K) * 4 + 72 * 4, (hipStream_t)stream>>>(y, pos, scores, sscore, res,
+                                                                                                    w, eps, h, xq, xs, M, K, topk);
+    else
+        moe_combine_kernel<4><<<dim3(Mp), dim3(NT), size_t(K) * 4 + 72 * 4, (hipStream_t)stream>>>(y, pos, scores, sscore, res,
+                                                                                                    w, eps, h, xq, xs, M, K, topk);
     return check_launch("moe_combine");
 }
 
