@@ -253,6 +253,81 @@ __global__ __launch_bounds__(NT) void qkv_headnorm_kernel(const int32_t* __restr
     }
 }
 
+// The same for head dim 128 and bf16 input on many rows: sixteen lanes per head with eight consecutive values each
+// (16-byte loads and stores, sixteen heads per pass of a workgroup) instead of a wave per head with two.  The sum of
+// squares is taken in the order of the kernel above, so both give the same bits: that one adds the squares of values
+// (2l, 2l + 1) in lane l and then runs a butterfly over lane distances 32, 16, 8, 4, 2, 1; here the lane keeps the four
+// pair sums of its eight values apart through the butterfly over group-lane distances 8, 4, 2, 1 (= 32 ... 4 there) and
+// joins them last, (p0 + p2) + (p1 + p3) (= distances 2 and 1).
+__global__ __launch_bounds__(NT) void qkv_headnorm128_kernel(const uint16_t* __restrict__ y, const uint16_t* __restrict__ qn,
+                                                             const uint16_t* __restrict__ kn, float eps,
+                                                             uint16_t* __restrict__ q, uint16_t* __restrict__ k,
+                                                             uint16_t* __restrict__ v, int L, int hq, int hk,
+                                                             const RopeArgs rope) {
+    constexpr int d = 128, U = 2, GROUPS = NT / 16;
+    const int row = blockIdx.x, grp = threadIdx.x >> 4, j = threadIdx.x & 15;
+    const int heads = hq + 2 * hk, ntot = heads * d;
+    const int64_t pos = rope.inv_freq ? (rope.pos_dev ? rope.pos_dev[0] : rope.pos0) + row : row;
+    const int kv_rows = rope.inv_freq ? rope.kv_rows : L;
+    __shared__ float s_sin[d / 2], s_cos[d / 2];
+    if (rope.inv_freq) {
+        if (threadIdx.x < d / 2) sincosf(float(pos) * rope.inv_freq[threadIdx.x], &s_sin[threadIdx.x], &s_cos[threadIdx.x]);
+        __syncthreads();
+    }
+    for (int g0 = grp; g0 < heads; g0 += U * GROUPS) {
+        u32x4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int g = g0 + u * GROUPS;
+            if (g < heads) raw[u] = *reinterpret_cast<const u32x4*>(y + size_t(row) * ntot + g * d + 8 * j);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int g = g0 + u * GROUPS;
+            if (g >= heads) break;
+            uint16_t* out;
+            int hh;
+            if (g < hq) { out = q; hh = g; } else if (g < hq + hk) { out = k; hh = g - hq; } else { out = v; hh = g - hq - hk; }
+            uint16_t* o = g >= hq              ? out + (size_t(hh) * kv_rows + size_t(pos)) * d + 8 * j
+                          : rope.q_token_major ? out + (size_t(row) * hq + hh) * d + 8 * j
+                                               : out + (size_t(hh) * L + row) * d + 8 * j;
+            if (g >= hq + hk) {   // v: as it is
+                *reinterpret_cast<u32x4*>(o) = raw[u];
+                continue;
+            }
+            float x[8], p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                x[2 * i] = __uint_as_float(raw[u][i] << 16);
+                x[2 * i + 1] = __uint_as_float(raw[u][i] & 0xFFFF0000u);
+                p[i] = __fadd_rn(__fmul_rn(x[2 * i], x[2 * i]), __fmul_rn(x[2 * i + 1], x[2 * i + 1]));
+            }
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) p[i] = __fadd_rn(p[i], __shfl_xor(p[i], off, 16));
+            const float ss = __fadd_rn(__fadd_rn(p[0], p[2]), __fadd_rn(p[1], p[3]));
+            const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, float(d)), eps)));
+            const u32x4 wr = *reinterpret_cast<const u32x4*>((g < hq ? qn : kn) + 8 * j);
+            u32x4 res;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float wv = __uint_as_float(i & 1 ? (wr[i >> 1] & 0xFFFF0000u) : (wr[i >> 1] << 16));
+                float nv = round_bf16(__fmul_rn(wv, round_bf16(__fmul_rn(x[i], inv))));
+                if (rope.inv_freq) {   // element 8 j + i pairs with the one 64 away, eight group lanes off
+                    const float other = __shfl_xor(nv, 8, 16);
+                    const int e = (8 * j + i) & 63;
+                    nv = j < 8 ? __fsub_rn(__fmul_rn(nv, s_cos[e]), __fmul_rn(other, s_sin[e]))
+                               : __fadd_rn(__fmul_rn(nv, s_cos[e]), __fmul_rn(other, s_sin[e]));
+                }
+                const uint32_t b = f32_to_bf16(nv);
+                if (i & 1) res[i >> 1] |= b << 16; else res[i >> 1] = b;
+            }
+            *reinterpret_cast<u32x4*>(o) = res;
+        }
+    }
+}
+
 // ---- OLMoE q/k/v split with RMSNorm over the full h*d width ------------------------------------------------------
 __global__ __launch_bounds__(NT) void qkv_fullnorm_kernel(const uint16_t* __restrict__ y, const uint16_t* __restrict__ qn,
                                                           const uint16_t* __restrict__ kn, float eps, uint16_t* __restrict__ q,
@@ -604,6 +679,14 @@ static dim3 headnorm_grid(int L, int heads) {
     return dim3(L, L >= 256 ? 1 : groups);
 }
 
+// Many rows of bf16 input with head dim 128 and 16-byte aligned operands take the kernel with 16-byte accesses (a few rows
+// are spread over more workgroups by the general one).
+static bool headnorm128_fits(const int32_t* acc, const uint16_t* y, const uint16_t* qn, const uint16_t* kn, const uint16_t* q,
+                             const uint16_t* k, const uint16_t* v, int L, int d) {
+    return !acc && d == 128 && L >= 16 &&
+           (uintptr_t(y) | uintptr_t(qn) | uintptr_t(kn) | uintptr_t(q) | uintptr_t(k) | uintptr_t(v)) % 16 == 0;
+}
+
 int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* y,
                       const uint16_t* qn, const uint16_t* kn, float eps, uint16_t* q, uint16_t* k, uint16_t* v, int L,
                       int hq, int hk, int d, void* stream) {
@@ -616,6 +699,11 @@ int scmx_qkv_headnorm(const int32_t* acc, const float* xscale, const float* wsca
         return SCMX_ERR_ARG;
     }
     if (L == 0) return SCMX_OK;
+    if (headnorm128_fits(acc, y, qn, kn, q, k, v, L, d)) {
+        qkv_headnorm128_kernel<<<dim3(L), dim3(NT), 0, (hipStream_t)stream>>>(y, qn, kn, eps, q, k, v, L, hq, hk,
+                                                                               RopeArgs{nullptr, nullptr, 0, 0, 0});
+        return check_launch("qkv_headnorm");
+    }
     qkv_headnorm_kernel<<<headnorm_grid(L, hq + 2 * hk), dim3(NT), 0, (hipStream_t)stream>>>(
         acc, xscale, wscale, y, qn, kn, eps, q, k, v, L, hq, hk, d, RopeArgs{nullptr, nullptr, 0, 0, 0});
     return check_launch("qkv_headnorm");
@@ -639,6 +727,11 @@ int scmx_qkv_headnorm_rope(const int32_t* acc, const float* xscale, const float*
         return SCMX_ERR_ARG;
     }
     if (L == 0) return SCMX_OK;
+    if (headnorm128_fits(acc, y, qn, kn, q, kcache, vcache, L, d)) {
+        qkv_headnorm128_kernel<<<dim3(L), dim3(NT), 0, (hipStream_t)stream>>>(
+            y, qn, kn, eps, q, kcache, vcache, L, hq, hk, RopeArgs{inv_freq, pos_dev, pos0, cache_rows, q_token_major});
+        return check_launch("qkv_headnorm_rope");
+    }
     qkv_headnorm_kernel<<<headnorm_grid(L, hq + 2 * hk), dim3(NT), 0, (hipStream_t)stream>>>(
         acc, xscale, wscale, y, qn, kn, eps, q, kcache, vcache, L, hq, hk, d, RopeArgs{inv_freq, pos_dev, pos0, cache_rows, q_token_major});
     return check_launch("qkv_headnorm_rope");

@@ -237,6 +237,33 @@ def test_fused_headnorm_rope_append_against_separate_ops(L, pos, from_acc):
         S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc, vc, rows - L + 1, inv_freq, **kw)
 
 
+def test_headnorm_rope_many_rows_equal_few_rows_at_a_time():
+    """Head dim 128 on many rows runs a kernel with sixteen lanes per head; a few rows run the general one (a wave per
+    head).  Both must give the same bits: 70 rows at once against the same rows eight at a time, q and both caches,
+    with the rotary embedding and (dense outputs) without."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    hq, hk, d, rows, L, pos = 16, 8, 128, 128, 70, 9
+    g = torch.Generator(device="cuda").manual_seed(3)
+    n = (hq + 2 * hk) * d
+    qn = (1 + 0.1 * torch.randn(d, device="cuda", generator=g)).to(torch.bfloat16)
+    kn = (1 + 0.1 * torch.randn(d, device="cuda", generator=g)).to(torch.bfloat16)
+    inv_freq = 1.0 / (1e6 ** (torch.arange(d // 2, device="cuda", dtype=torch.float32) / (d // 2)))
+    y = (torch.randn(L, n, device="cuda", generator=g) * torch.rand(L, 1, device="cuda", generator=g) * 4).to(torch.bfloat16)
+    kc, vc = (torch.zeros((hk, rows, d), device="cuda", dtype=torch.bfloat16) for _ in range(2))
+    q = S.qkv_headnorm_rope(y, qn, kn, 1e-6, L, hq, hk, d, kc, vc, pos, inv_freq)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    for r0 in range(0, L, 8):
+        r1 = min(L, r0 + 8)
+        qp = S.qkv_headnorm_rope(y[r0:r1].contiguous(), qn, kn, 1e-6, r1 - r0, hq, hk, d, kc2, vc2, pos + r0, inv_freq)
+        assert torch.equal(qp, q[:, r0:r1])
+    assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    q0, k0, v0 = S.qkv_headnorm_y(y, qn, kn, 1e-6, L, hq, hk, d)
+    for r0 in range(0, L, 8):
+        r1 = min(L, r0 + 8)
+        qp, kp, vp = S.qkv_headnorm_y(y[r0:r1].contiguous(), qn, kn, 1e-6, r1 - r0, hq, hk, d)
+        assert torch.equal(qp, q0[:, r0:r1]) and torch.equal(kp, k0[:, r0:r1]) and torch.equal(vp, v0[:, r0:r1])
+
+
 @pytest.mark.parametrize("hq,hk,d,rows,n", [(16, 8, 128, 512, 129), (4, 4, 64, 40, 1), (8, 2, 256, 300, 300), (16, 8, 128, 8192, 5000),
                                             (16, 8, 128, 4096, 3000)])
 def test_attn_decode_against_torch(hq, hk, d, rows, n):
