@@ -113,6 +113,94 @@ __global__ __launch_bounds__(NT) void rmsnorm_quant_kernel(const uint16_t* __res
     block_quant_row(srow, K, qrow, xs + row, red);
 }
 
+// The same with the row in registers: one wave per row, lane l owns the 16-byte pieces l, l + 64, ... (CH of them,
+// K = 512 * CH), four rows per workgroup, no LDS and no workgroup barrier.  The sum of squares is taken in the order of
+// block_inv_rms, so both kernels give the same bits: there, thread (wave g, lane t) adds the squares of elements
+// 256 g + 4 t .. + 3 in sequence, a butterfly over lane distances 32 ... 1 gives the sum of group g, and a second
+// butterfly over the group sums (zeros beyond the last group) gives the total.  Here piece l + 64 j holds the
+// elements of lanes 2 (l % 32) and 2 (l % 32) + 1 of group 2 j + l / 32: the two four-element sums stay apart through
+// the butterfly over lane distances 16 ... 1 (= 32 ... 2 there) and are added last (= distance 1); lane l then picks
+// up the sum of group l and the second butterfly runs as it does there.
+template <int CH>
+__global__ __launch_bounds__(256) void rmsnorm_quant_wave_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                                 float eps, int8_t* __restrict__ xq, float* __restrict__ xs,
+                                                                 uint16_t* __restrict__ xn, int M, int Mp) {
+    constexpr int K = 512 * CH;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= Mp) return;
+    u32x2* qrow = reinterpret_cast<u32x2*>(xq + size_t(row) * K);
+    u32x4* nrow = xn ? reinterpret_cast<u32x4*>(xn + size_t(row) * K) : nullptr;
+    if (row >= M) {
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            qrow[lane + 64 * j] = u32x2{0u, 0u};
+            if (nrow) nrow[lane + 64 * j] = u32x4{0u, 0u, 0u, 0u};
+        }
+        if (lane == 0) xs[row] = 0.0f;
+        return;
+    }
+    const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
+    const u32x4* wrow = reinterpret_cast<const u32x4*>(w);
+    u32x4 v[CH], wv[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) v[j] = xrow[lane + 64 * j];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) wv[j] = wrow[lane + 64 * j];
+    auto lo = [](uint32_t u) { return __uint_as_float(u << 16); };
+    auto hi = [](uint32_t u) { return __uint_as_float(u & 0xFFFF0000u); };
+    float r = 0.0f;   // lane l < 2 CH: the sum of group l
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+        float a = __fmul_rn(lo(v[j][0]), lo(v[j][0]));
+        a = __fadd_rn(a, __fmul_rn(hi(v[j][0]), hi(v[j][0])));
+        a = __fadd_rn(a, __fmul_rn(lo(v[j][1]), lo(v[j][1])));
+        a = __fadd_rn(a, __fmul_rn(hi(v[j][1]), hi(v[j][1])));
+        float b = __fmul_rn(lo(v[j][2]), lo(v[j][2]));
+        b = __fadd_rn(b, __fmul_rn(hi(v[j][2]), hi(v[j][2])));
+        b = __fadd_rn(b, __fmul_rn(lo(v[j][3]), lo(v[j][3])));
+        b = __fadd_rn(b, __fmul_rn(hi(v[j][3]), hi(v[j][3])));
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) {
+            a = __fadd_rn(a, __shfl_xor(a, off, WAVE));
+            b = __fadd_rn(b, __shfl_xor(b, off, WAVE));
+        }
+        const float mine = __fadd_rn(a, b);                 // group 2 j + lane / 32
+        const float other = __shfl_xor(mine, 32, WAVE);     // the other group of this j
+        const float even = lane < 32 ? mine : other, odd = lane < 32 ? other : mine;
+        if ((lane >> 1) == j) r = (lane & 1) ? odd : even;
+    }
+    const float tot = wave_sum(r);
+    const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(tot, float(K)), eps)));
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float n0 = round_bf16(__fmul_rn(lo(wv[j][e]), round_bf16(__fmul_rn(lo(v[j][e]), inv))));
+            const float n1 = round_bf16(__fmul_rn(hi(wv[j][e]), round_bf16(__fmul_rn(hi(v[j][e]), inv))));
+            amax = fmaxf(amax, fmaxf(fabsf(n0), fabsf(n1)));
+            v[j][e] = (__float_as_uint(n0) >> 16) | (__float_as_uint(n1) & 0xFFFF0000u);
+        }
+        if (nrow) nrow[lane + 64 * j] = v[j];
+    }
+    amax = wave_max(amax);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+        uint32_t o[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int q0 = quant_code(lo(v[j][e]), qi);
+            const int q1 = quant_code(hi(v[j][e]), qi);
+            o[e >> 1] |= (uint32_t(q0) & 0xFFu) << (16 * (e & 1));
+            o[e >> 1] |= (uint32_t(q1) & 0xFFu) << (16 * (e & 1) + 8);
+        }
+        qrow[lane + 64 * j] = u32x2{o[0], o[1]};
+    }
+    if (lane == 0) xs[row] = s;
+}
+
 // ---- res_norm_quant / res_epilogue -----------------------------------------------------------------------------
 __global__ __launch_bounds__(NT) void res_norm_quant_kernel(const int32_t* __restrict__ acc, const float* __restrict__ xscale,
                                                             const float* __restrict__ wscale, const uint16_t* __restrict__ res,
@@ -640,7 +728,23 @@ int scmx_rmsnorm_quant(const uint16_t* x, const uint16_t* w, float eps, int8_t* 
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
-    rmsnorm_quant_kernel<<<dim3(Mp), dim3(NT), size_t(K) * 2 + 72 * 4, (hipStream_t)stream>>>(x, w, eps, xq, xs, xn, M, K);
+    hipStream_t st = (hipStream_t)stream;
+    if (K % 512 == 0 && (uintptr_t(x) | uintptr_t(w) | uintptr_t(xn)) % 16 == 0 && uintptr_t(xq) % 8 == 0) {
+        // rows of up to 4096 elements stay in registers (one wave per row)
+        const dim3 wgrid((Mp + 3) / 4), block(256);
+        switch (K / 512) {
+            case 1: rmsnorm_quant_wave_kernel<1><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 2: rmsnorm_quant_wave_kernel<2><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 3: rmsnorm_quant_wave_kernel<3><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 4: rmsnorm_quant_wave_kernel<4><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 5: rmsnorm_quant_wave_kernel<5><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 6: rmsnorm_quant_wave_kernel<6><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 7: rmsnorm_quant_wave_kernel<7><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            case 8: rmsnorm_quant_wave_kernel<8><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
+            default: break;
+        }
+    }
+    rmsnorm_quant_kernel<<<dim3(Mp), dim3(NT), size_t(K) * 2 + 72 * 4, st>>>(x, w, eps, xq, xs, xn, M, K);
     return check_launch("rmsnorm_quant");
 }
 

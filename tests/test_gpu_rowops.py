@@ -18,7 +18,8 @@ def S():
     return sc_kernels
 
 
-@pytest.mark.parametrize("m,k", [(200, 2048), (3, 128), (65, 4096), (9, 1000)])
+@pytest.mark.parametrize("m,k", [(200, 2048), (3, 128), (65, 4096), (9, 1000), (70, 512), (33, 1536), (5, 3584), (2048, 2048),
+                                 (130, 6144)])
 def test_rmsnorm_quant(S, m, k):
     rng = np.random.default_rng(k + m)
     x = bf16.to_bits((rng.standard_normal((m, k)) * rng.lognormal(0, 1, (1, k))).astype(F32))
