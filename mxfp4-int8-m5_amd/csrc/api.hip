@@ -404,7 +404,7 @@ int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int 
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
-    const dim3 wgrid((Mp + 3) / 4), block(256);
+    const dim3 wgrid((unsigned(Mp) + 3u) / 4u), block(256);
     hipStream_t st = (hipStream_t)stream;
     switch (K % 512 ? 0 : K / 512) {   // rows of up to 8192 elements stay in registers
         case 1: act_quant_wave_kernel<1><<<wgrid, block, 0, st>>>(x, xq, xs, M, Mp); break;

@@ -731,7 +731,7 @@ int scmx_rmsnorm_quant(const uint16_t* x, const uint16_t* w, float eps, int8_t* 
     hipStream_t st = (hipStream_t)stream;
     if (K % 512 == 0 && (uintptr_t(x) | uintptr_t(w) | uintptr_t(xn)) % 16 == 0 && uintptr_t(xq) % 8 == 0) {
         // rows of up to 4096 elements stay in registers (one wave per row)
-        const dim3 wgrid((Mp + 3) / 4), block(256);
+        const dim3 wgrid((unsigned(Mp) + 3u) / 4u), block(256);
         switch (K / 512) {
             case 1: rmsnorm_quant_wave_kernel<1><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
             case 2: rmsnorm_quant_wave_kernel<2><<<wgrid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); return check_launch("rmsnorm_quant");
