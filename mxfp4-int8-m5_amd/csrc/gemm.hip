@@ -853,6 +853,19 @@ static int packed_mode(const DevFormat& f) {
 static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     const long cus = device_cus();
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
+#ifdef SCMX_TUNE
+    if (const char* e = getenv("SCMX_TILE")) {
+        switch (atoi(e)) {
+            case 0: return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
+            case 1: return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
+            case 2: return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
+
+            case 4: return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
+            case 5: return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
+            case 6: if (a.K % 256 == 0) return launch_tile<64, 64, 128, 2, 2, 1, 2, false, false, 2>(a, bmode, (a.M + 63) / 64, s); break;
+        }
+    }
+#endif
     // The tile is the one a small cost model makes fastest.  A launch runs its tiles in waves of (CUs x workgroups that
     // share a CU); a wave costs F + S per 128 of K and not less than W, all three measured per configuration and per
     // number of co-resident workgroups (four Qwen3-1.7B layer shapes and five others, K = 128 ... 6144, M = 64 ... 8192:
@@ -860,27 +873,31 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     // faster (less contention for the L2s and HBM).  What the table encodes: 256x256 moves the fewest LDS bytes per MFMA
     // and pays where it fills the chip or saves a round; a mostly empty last round costs more than a narrower tile's
     // extra LDS traffic; the small tiles share a CU and lose less to a ragged tile count; with no more 64x64 tiles
-    // than CUs two K groups per tile put eight waves on a CU.  (A 256x64 tile was never the fastest and is gone.)
+    // than CUs two K groups per tile put eight waves on a CU, and with no more 64x32 tiles than CUs four K groups of two
+    // waves do (a 2048-wide layer on up to 128 rows: 64 ... 128 tiles instead of 32 ... 64; down 14.4 -> 10.2-10.9 us).
+    // (A 256x64 tile was never the fastest and is gone.)
     struct Cand {
         int bm, bn, occ;
         float f[3], s[3], w[3];   // per wave, by co-resident workgroups 1..occ: fixed us, us per 128 of K, least us
         float low, mid;           // a wave on half of the CUs or fewer / on three quarters of them costs this part of a full one
     };
-    static const Cand cand[6] = {
+    static const Cand cand[7] = {
         {256, 256, 1, {6.5f, 0, 0}, {1.9f, 0, 0}, {8.4f, 0, 0}, 0.70f, 0.835f},
         {256, 128, 1, {4.2f, 0, 0}, {0.94f, 0, 0}, {5.5f, 0, 0}, 0.74f, 0.78f},
         {128, 128, 1, {1.4f, 0, 0}, {0.62f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
         {128, 64, 2, {1.4f, 1.2f, 0}, {0.39f, 0.77f, 0}, {2.2f, 3.0f, 0}, 0.91f, 1.0f},
         {64, 64, 3, {0.85f, 0.6f, 0.6f}, {0.34f, 0.53f, 0.70f}, {1.9f, 2.3f, 2.7f}, 0.95f, 1.0f},
         {64, 64, 1, {1.1f, 0, 0}, {0.26f, 0, 0}, {2.0f, 0, 0}, 0.97f, 1.0f},   // two K groups
+        {64, 32, 1, {1.26f, 0, 0}, {0.14f, 0, 0}, {2.0f, 0, 0}, 0.95f, 0.97f},  // four K groups
     };
     const float steps = float(a.K) / 128.0f;
     int best = 4;
     float best_t = 1e30f;
-    for (int c = 0; c < 6; ++c) {
+    for (int c = 0; c < 7; ++c) {
         const Cand& k = cand[c];
         const long n = tiles(k.bm, k.bn);
         if (c == 5 && (n > cus || a.K % 256)) continue;
+        if (c == 6 && (n > cus || a.K % 512)) continue;
         const long cap = cus * k.occ;
         const long full = n / cap, rest = n % cap;
         float t = float(full) * fmaxf(k.f[k.occ - 1] + steps * k.s[k.occ - 1], k.w[k.occ - 1]);
@@ -906,6 +923,7 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
         case 2: return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
         case 3: return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
         case 5: return launch_tile<64, 64, 128, 2, 2, 1, 2, false, false, 2>(a, bmode, (a.M + 63) / 64, s);
+        case 6: return launch_tile<64, 32, 128, 2, 1, 1, 2, false, false, 4>(a, bmode, (a.M + 63) / 64, s);
         default: return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
     }
 }

@@ -327,12 +327,13 @@ def test_config1_m512_and_m8192_against_the_oracle(S, name, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(512, 2048, 6144), (131, 2048, 2048), (192, 4096, 1024), (16, 256, 1024), (200, 1000, 1280),
-                                   (64, 16384, 768)])
+                                   (64, 16384, 768), (100, 2048, 6144), (3, 8, 512)])
 @pytest.mark.parametrize("fmt_i", [0, 1, 2, 5])
 def test_few_tiles_two_k_groups(S, m, n, k, fmt_i):
-    """Problems with no more 64x64 tiles than CUs and enough K steps run two K groups per tile whose INT32 partial sums
-    meet in LDS: INT32 output and every epilogue against the oracle, from three K steps per group to 24, in four
-    formats (one per decode path of the kernel), from INT8 and from packed weights."""
+    """Problems with no more 64x64 tiles than CUs run two K groups per tile, with no more 64x32 tiles than CUs (and K a
+    multiple of 512) four, whose INT32 partial sums meet in LDS: INT32 output and every epilogue against the oracle,
+    from one K step per group to 24, in four formats (one per decode path of the kernel), from INT8 and from packed
+    weights."""
     fmt = FORMATS[fmt_i]
     rng = np.random.default_rng(m + n + k + fmt_i)
     codes, bc, _, q = random_packed(rng, n, k, fmt)
