@@ -848,24 +848,10 @@ static int packed_mode(const DevFormat& f) {
                                         : B_PACKED_GENERIC;
 }
 
-// Dense: the largest tile that still gives every CU a workgroup.  256x256 (wave tiles of 128x64, K steps of 64) moves
-// 25 % fewer LDS bytes per MFMA than 256x128 and is worth 4-5 % where the problem has 256 such tiles.
+// Dense: one launch, with the tile a cost model of the candidates below makes fastest.
 static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
     const long cus = device_cus();
     auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-#ifdef SCMX_TUNE
-    if (const char* e = getenv("SCMX_TILE")) {
-        switch (atoi(e)) {
-            case 0: return launch_tile<256, 256, 64, 2, 4, 1, 2>(a, bmode, (a.M + 255) / 256, s);
-            case 1: return launch_tile<256, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 255) / 256, s);
-            case 2: return launch_tile<128, 128, 128, 4, 2, 1, 3>(a, bmode, (a.M + 127) / 128, s);
-
-            case 4: return launch_tile<128, 64, 128, 4, 2>(a, bmode, (a.M + 127) / 128, s);
-            case 5: return launch_tile<64, 64, 128, 2, 2>(a, bmode, (a.M + 63) / 64, s);
-            case 6: if (a.K % 256 == 0) return launch_tile<64, 64, 128, 2, 2, 1, 2, false, false, 2>(a, bmode, (a.M + 63) / 64, s); break;
-        }
-    }
-#endif
     // The tile is the one a small cost model makes fastest.  A launch runs its tiles in waves of (CUs x workgroups that
     // share a CU); a wave costs F + S per 128 of K and not less than W, all three measured per configuration and per
     // number of co-resident workgroups (four Qwen3-1.7B layer shapes and five others, K = 128 ... 6144, M = 64 ... 8192:
