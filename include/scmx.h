@@ -81,6 +81,12 @@ int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t*
  * Replaces act_quant, e2e/sc_kernels.py:200-229,554-563. */
 int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream);
 
+/* scmx_act_quant (e2e/sc_kernels.py:200-229) writing xq in the BLOCKED layout that scmx_mm_w4a8_blocked reads: blocks
+ * of 32 rows x 32 k (1 KB each), block (m / 32, k / 32) at byte ((m / 32) * (K / 32) + k / 32) * 1024, and inside a block
+ * the 16 bytes xq[m, 16 j .. 16 j + 15] (j = k / 16) at ((j % 2) * 32 + m % 32) * 16.  Same codes and scales as
+ * scmx_act_quant.  Mp % 32 == 0, K % 32 == 0; xq holds Mp * K bytes, rows >= M are zero with scale 0. */
+int scmx_act_quant_blocked(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream);
+
 /* INT8 [M,K] x INT8 [N,K]^T -> INT32 [M,N] on INT8 MFMA.  Replaces mm_i8_i32, e2e/sc_kernels.py:53-71,486-495. */
 int scmx_mm_i8_i32(const int8_t* xq, const int8_t* wq, int32_t* acc, int M, int N, int K, void* stream);
 
@@ -97,7 +103,16 @@ int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, 
                  const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M, int N,
                  int K, void* stream);
 
-/* Whole dense W4A8 linear on a bf16 input: activation quantization prologue + scmx_mm_w4a8, one call.
+/* scmx_mm_w4a8 on activations in the blocked layout of scmx_act_quant_blocked (xq: ceil(M / 32) * 32 rows, 16-byte
+ * aligned): the waves of the large tiles load their activation fragments straight from memory, and only the weights
+ * pass through LDS.  Same results as scmx_mm_w4a8 (same integers, same epilogues).  Meant for prefill-sized M: every
+ * shape runs, on 128x128 tiles at least.  The same pair of reference calls as scmx_mm_w4a8 (e2e/fused_qwen3.py:161-172). */
+int scmx_mm_w4a8_blocked(const scmx_format* fmt, const int8_t* xq, const float* xscale, const uint32_t* codes,
+                         const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M,
+                         int N, int K, void* stream);
+
+/* Whole dense W4A8 linear on a bf16 input: activation quantization prologue + scmx_mm_w4a8, one call (the activations
+ * are quantized into the blocked layout when the shape runs on a tile that reads it).
  * workspace must hold scmx_linear_w4a8_workspace(M, K) bytes (the INT8 activations and their scales). */
 size_t scmx_linear_w4a8_workspace(int M, int K);
 int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* codes, const uint8_t* bcodes,

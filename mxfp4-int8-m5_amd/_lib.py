@@ -26,9 +26,11 @@ SIGNATURES = {
     "scmx_mxfp4_format": (None, [_FMT]),
     "scmx_unpack_i8": (_I, [_FMT, _P, _P, _P, _L, _L, _P]),
     "scmx_act_quant": (_I, [_P, _P, _P, _I, _I, _I, _P]),
+    "scmx_act_quant_blocked": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "scmx_mm_i8_i32": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "scmx_mm_epi": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_mm_w4a8": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "scmx_mm_w4a8_blocked": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_linear_w4a8_workspace": (_Z, [_I, _I]),
     "scmx_linear_w4a8": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "scmx_linear_w4a8_static_max_elements": (_Z, []),

@@ -240,6 +240,80 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(const uint16_t* __r
     if (lane == 0) xs[row] = s;
 }
 
+// ---- act_quant into the blocked layout ---------------------------------------------------------------------------
+// xq as the large dense GEMM tiles take it: blocks of 32 rows x 32 k (1 KB), block (m / 32, k / 32) at
+// ((m / 32) * (K / 32) + k / 32) KB, and inside a block the 16 bytes of row r, k half h at (32 h + r) * 16 -- the order
+// in which the 64 lanes of a wave hold a 32x32x32 MFMA operand, so that a wave fetches one block with one coalesced load.
+// One wave per row, the row in registers (NJ > 0: K = 1024 NJ, lane l owns the 16-element pieces l, l + 64, ...) or read
+// twice (NJ = 0: any K % 32 == 0); eight rows per workgroup, which between them write whole 128-byte lines.  Same codes
+// and scales as act_quant_kernel: the row maximum does not depend on the order it is taken in.
+template <int NJ>
+__global__ __launch_bounds__(512) void act_quant_blocked_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
+                                                                float* __restrict__ xs, int M, int Mp, int K) {
+    const int row = blockIdx.x * 8 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= Mp) return;
+    if (NJ > 0) K = 1024 * NJ;
+    const int pieces = K / 16;
+    // piece c of the row (k = 16 c ...): k slice c / 2, half c % 2
+    int8_t* const dst = xq + (size_t(row >> 5) * size_t(K >> 5)) * 1024 + size_t(row & 31) * 16;
+    auto at = [&](int c) { return reinterpret_cast<u32x4*>(dst + size_t(c >> 1) * 1024 + (c & 1) * 512); };
+    if (row >= M) {
+        for (int c = lane; c < pieces; c += 64) *at(c) = u32x4{0u, 0u, 0u, 0u};
+        if (lane == 0) xs[row] = 0.0f;
+        return;
+    }
+    const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
+    auto amax8 = [](const u32x4& v, float m) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            m = fmaxf(m, fabsf(__uint_as_float(v[e] << 16)));
+            m = fmaxf(m, fabsf(__uint_as_float(v[e] & 0xFFFF0000u)));
+        }
+        return m;
+    };
+    auto codes8 = [](const u32x4& v, float qi) {
+        uint32_t o[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int q0 = quant_code(__uint_as_float(v[e] << 16), qi);
+            const int q1 = quant_code(__uint_as_float(v[e] & 0xFFFF0000u), qi);
+            o[e >> 1] |= (uint32_t(q0) & 0xFFu) << (16 * (e & 1));
+            o[e >> 1] |= (uint32_t(q1) & 0xFFu) << (16 * (e & 1) + 8);
+        }
+        return u32x2{o[0], o[1]};
+    };
+    constexpr int NR = NJ > 0 ? NJ : 1;
+    u32x4 v[NR][2];
+    float amax = 0.0f;
+    if (NJ > 0) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            v[j][0] = xrow[2 * (lane + 64 * j)];
+            v[j][1] = xrow[2 * (lane + 64 * j) + 1];
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) amax = amax8(v[j][1], amax8(v[j][0], amax));
+    } else {
+        for (int c = lane; c < pieces; c += 64) amax = amax8(xrow[2 * c + 1], amax8(xrow[2 * c], amax));
+    }
+    amax = wave_max(amax);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+    if (NJ > 0) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const u32x2 lo = codes8(v[j][0], qi), hi = codes8(v[j][1], qi);
+            *at(lane + 64 * j) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    } else {
+        for (int c = lane; c < pieces; c += 64) {
+            const u32x2 lo = codes8(xrow[2 * c], qi), hi = codes8(xrow[2 * c + 1], qi);
+            *at(c) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    }
+    if (lane == 0) xs[row] = s;
+}
+
 // ---- rot_quant: randomized Hadamard rotation of every 32-wide block, then per-token INT8 ---------------------------
 // Thread t owns 4 consecutive values; 8 consecutive lanes hold one block.  Butterfly order as in the host
 // formulation: two stages inside the thread, then strides 1, 2, 4 across lanes (lower = lower + upper,
@@ -396,6 +470,28 @@ int scmx_unpack_i8(const scmx_format* fmt, const uint32_t* codes, const uint8_t*
             f, codes, bcodes, (u32x2*)wq, words, int(K / 8), bc_row_bytes);
     }
     return check_launch("unpack_i8");
+}
+
+int scmx_act_quant_blocked(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream) {
+    if (!x || !xq || !xs || M < 0 || Mp < M || Mp % 32 || Mp > (1 << 30) || K <= 0 || K % 32 || uintptr_t(x) % 16 ||
+        uintptr_t(xq) % 16) {
+        set_error("act_quant_blocked: need M <= Mp <= 2^30 with Mp %% 32 == 0 (Mp = %d), K %% 32 == 0 (K = %d), x and xq "
+                  "16-byte aligned", Mp, K);
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    const dim3 grid((unsigned(Mp) + 7u) / 8u), block(512);
+    hipStream_t st = (hipStream_t)stream;
+    switch (K % 1024 ? 0 : K / 1024) {   // rows of up to 8192 elements stay in registers
+        case 1: act_quant_blocked_kernel<1><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+        case 2: act_quant_blocked_kernel<2><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+        case 3: act_quant_blocked_kernel<3><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+        case 4: act_quant_blocked_kernel<4><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+        case 6: act_quant_blocked_kernel<6><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+        case 8: act_quant_blocked_kernel<8><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+        default: act_quant_blocked_kernel<0><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+    }
+    return check_launch("act_quant_blocked");
 }
 
 int scmx_act_quant(const uint16_t* x, int8_t* xq, float* xs, int M, int Mp, int K, void* stream) {

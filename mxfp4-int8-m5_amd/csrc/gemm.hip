@@ -16,7 +16,7 @@
 namespace scmx {
 
 struct GemmArgs {
-    const int8_t* xq;        // activations INT8 [rows, K]
+    const int8_t* xq;        // activations INT8 [rows, K] (blocked: 32 x 32 blocks in MFMA operand order, see AD)
     const float* xscale;     // [rows]
     const int32_t* gather;   // optional: logical row r reads xq[gather[r]], xscale[gather[r]]
     const uint32_t* codes;   // packed weights [E][N*K/8]
@@ -32,6 +32,7 @@ struct GemmArgs {
     const uint16_t* silu;    // SwiGLU epilogue: lookup table over bf16 gate values
     const int32_t* tstart;   // grouped: first row tile of each expert [E+1]
     int n_experts;
+    int blocked;             // dense: xq is in the blocked layout
     DevFormat fmt;
 };
 
@@ -54,7 +55,7 @@ enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3,
 // K / KG of the reduction out of LDS stages of its own, and the INT32 partial sums meet in LDS before the epilogue (exact:
 // integer addition is associative).  A CU then runs KG times the waves on the same tile count.
 template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false,
-          int KG = 1>
+          int KG = 1, bool AD = false>
 __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const GemmArgs a) {
     constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
     constexpr int NT = WGM * WGN * 64;   // threads of one K group
@@ -63,8 +64,9 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && (BK == 64 || BK == 128), "tile must be whole 32x32x32 MFMAs");
     constexpr int CPR = BK / 16;             // 16-byte chunks per LDS row
     constexpr int RPB = 256 / BK;            // rows per 256 bytes, i.e. per sweep of the 64 LDS banks
-    constexpr int A_CHUNKS = BM * CPR;       // 16-byte pieces of the activation tile
-    constexpr int A_PER = (A_CHUNKS + NT - 1) / NT;
+    constexpr int A_CHUNKS = AD ? 0 : BM * CPR;   // 16-byte pieces of the activation tile
+    constexpr int A_PER = AD ? 1 : (A_CHUNKS + NT - 1) / NT;
+    constexpr int A_BYTES = AD ? 0 : BM * BK;     // the activation rows of a stage
     // packed weights are staged in runs of 8 * WPC weights (WPC code words) per thread: 32 when that keeps every
     // thread busy, else 16
     constexpr int WPC = BN * BK / 32 >= NT ? 4 : 2;
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     static_assert(!PK || (BK == 128 && WPC == 4 && (BMODE == B_PACKED_DEFAULT || BMODE == B_PACKED_B16)),
                   "packed weights in LDS: K steps of 128, 16-byte runs, FP4-conversion formats");
     // bytes per stage: BM activation rows, then BN weight rows (PK: 64 code bytes each)
-    constexpr int STAGE = BM * BK + (PK ? BN * (BK / 2) : BN * BK);
+    constexpr int STAGE = A_BYTES + (PK ? BN * (BK / 2) : BN * BK);
     static_assert(STAGE % 16 == 0, "stages keep 16-byte alignment");
 
     // Rows are BK bytes with no padding; the 16-byte chunk c of row r sits at chunk c ^ ((r / RPB) % CPR), which
@@ -83,6 +85,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     // need more than the stages and still fit the CU, the buffer is sized for them.
     constexpr int EPI_BYTES = WGM * WGN * WTM * (WTN * 2 + 16);
     static_assert(KG == 1 || (!PK && !SKIP), "K groups: staged dense tiles");
+    static_assert(!AD || (!PK && !SKIP && KG == 1), "activation fragments from memory: staged dense tiles");
     constexpr int GROUP_BYTES = NSTAGE * STAGE;
     // after the K loop: group 0's output tiles (the widest epilogue's) from 0, then the other groups' partial sums
     constexpr int PART_BYTES = NT * MI * NI * 64;
@@ -170,6 +173,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     uint32_t a_live = 0;   // SKIP: the chunks of rows inside the segment (the others are neither written to LDS nor used)
 #pragma unroll
     for (int j = 0; j < A_PER; ++j) {
+        if (AD) { a_src[j] = a_dst[j] = 0; continue; }
         const int c = tid + j * NT;
         const int row = c / CPR, kc = c % CPR;
         if (m0 + row < row_end) a_live |= 1u << j;
@@ -187,7 +191,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
             const int row = c / CPR, kc = c % CPR;
             const int gn = min(n0 + row, a.N - 1);
             b_src[j] = gn * K + kc * 16 + kbase;
-            b_dst[j] = BM * BK + swz(row, kc);
+            b_dst[j] = A_BYTES + swz(row, kc);
             b_dst2[j] = 0;
             b_bc[j] = 0;
             b_k[j] = 0;
@@ -205,11 +209,11 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                                                                         : 0);
             if (BMODE == B_PACKED_E8M0) b_rmin[j] = e8m0_row_min(a.wscale[erow + gn]);
             if (PK) {   // the run's 16 code bytes as they are
-                b_dst[j] = BM * BK + swzp(row, kb);
+                b_dst[j] = A_BYTES + swzp(row, kb);
                 b_dst2[j] = 0;
             } else {
-                b_dst[j] = BM * BK + swz(row, kb * WPC / 2);
-                b_dst2[j] = BM * BK + swz(row, kb * WPC / 2 + 1);
+                b_dst[j] = A_BYTES + swz(row, kb * WPC / 2);
+                b_dst2[j] = A_BYTES + swz(row, kb * WPC / 2 + 1);
             }
             b_k[j] = kb * 8 * WPC;
         }
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
     auto load_slice = [&](Staged& r, int k0, int q) {
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
-            if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS))
+            if (!AD && j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS))
                 r.a[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_src[j], k0, 0);
         if (q != NKK - 1) return;
 #pragma unroll
@@ -279,7 +283,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
         k0 += kbase;   // block indices below count from the row's first weight
 #pragma unroll
         for (int j = 0; j < A_PER; ++j)
-            if (j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS) && (!SKIP || ((a_live >> j) & 1u)))
+            if (!AD && j % NKK == q && (A_CHUNKS % NT == 0 || tid + j * NT < A_CHUNKS) && (!SKIP || ((a_live >> j) & 1u)))
                 *reinterpret_cast<u32x4*>(st + a_dst[j]) = r.a[j];
 #pragma unroll
         for (int j = 0; j < B_PER; ++j)
@@ -344,7 +348,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) koff[kk] = ((2 * kk + half) ^ sw) << 4;
     const int a_frag = (wm * WTM + lr) * BK;
-    const int b_frag = BM * BK + (wn * WTN + lr) * BK;
+    const int b_frag = A_BYTES + (wn * WTN + lr) * BK;
 
     const int KT = KL / BK;
     // Pipeline.  Iteration kt: barrier; multiply step kt out of its LDS stage while the register set holding step
@@ -403,7 +407,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
         koff_pa[kp][1] = ((4 * kp + 2 * half + 1) ^ sw) << 4;
         koff_pw[kp] = ((2 * kp + half) ^ ((lr >> 2) & 3)) << 4;
     }
-    [[maybe_unused]] const int w_frag = BM * BK + (wn * WTN + lr) * (BK / 2);
+    [[maybe_unused]] const int w_frag = A_BYTES + (wn * WTN + lr) * (BK / 2);
     auto load_pa = [&](const int8_t* src, int kp, v4i (&f)[2][MI]) {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
@@ -492,10 +496,36 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
         if (SKIP && mi_active == 0) return;
 #pragma unroll
         for (int i = 0; i < MI; ++i)
-            if (!SKIP || i < mi_active) xa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
+            if (!AD && (!SKIP || i < mi_active)) xa[i] = *reinterpret_cast<const v4i*>(src + a_frag + i * 32 * BK + koff[kk]);
 #pragma unroll
         for (int j = 0; j < NI; ++j) xb[j] = *reinterpret_cast<const v4i*>(src + b_frag + j * 32 * BK + koff[kk]);
     };
+    // AD: the activations come in 32-row x 32-k blocks of 1 KB laid out as the MFMA takes them (lane l = row l % 32,
+    // k half l / 32, 16 bytes each), block (m / 32, k / 32) at ((m / 32) * (K / 32) + k / 32) KB.  Every wave loads the
+    // fragments of its own rows straight into registers, two K steps ahead, in three buffers that rotate with the LDS
+    // stages: the activation tile never passes through LDS.
+    [[maybe_unused]] v4i fad[NSTAGE][NKK][MI];
+    [[maybe_unused]] int ad_src[MI];
+    if constexpr (AD) {
+        const int last_block = (a.M + 31) / 32 - 1;
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+            ad_src[i] = int(uint32_t(min((m0 + wm * WTM) / 32 + i, last_block)) * uint32_t(K >> 5) * 1024u + uint32_t(lane) * 16u +
+                            uint32_t(kbase) * 32u);
+    }
+    auto load_ad = [&](int buf, int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk)
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, ad_src[i] + kk * 1024, k0 * 32, 0);
+                fad[buf][kk][i] = v4i{int(v[0]), int(v[1]), int(v[2]), int(v[3])};
+            }
+    };
+    if constexpr (AD) {
+        load_ad(0, 0);
+        load_ad(1, min(BK, KL - BK));
+    }
     __syncthreads();
     if constexpr (PK) {
         load_pa(smem, 0, pa[0]);
@@ -522,6 +552,7 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
         const int k2 = min((kt + 2) * BK, KL - BK);      // past the end: rewrites a stage nobody reads again
         const int k4 = min((kt + 4) * BK, KL - BK);
         uint32_t o[B_PER][8];
+        if constexpr (AD && ST) load_ad(wr, k2);
 #pragma unroll
         for (int kk = 0; kk < NKK; ++kk) {
             if (kk + AHEAD < NKK)
@@ -534,7 +565,8 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
                 if (SKIP && i >= mi_active) continue;
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], fa[(ph + kk) % FD][i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], AD ? fad[rd][kk][i] : fa[(ph + kk) % FD][i],
+                                                                      acc[i][j], 0, 0, 0);
             }
             if constexpr (ST) stage_slice(r, dst, k2, kk, o);
             __builtin_amdgcn_sched_barrier(0);
@@ -812,7 +844,8 @@ __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const Gemm
 
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false, int KG = 1>
+template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false, int KG = 1,
+          bool AD = false>
 static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStream_t s) {
     GemmArgs a = a_in;
     if (a.epi == SCMX_EPI_SWIGLU) a.silu = silu_table_device();
@@ -826,17 +859,17 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
     } else {
         if (bmode == B_INT8)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_DEFAULT)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16M)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_E8M0)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP, false, KG><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
     }
 }
 
@@ -849,9 +882,11 @@ static int packed_mode(const DevFormat& f) {
 }
 
 // Dense: one launch, with the tile a cost model of the candidates below makes fastest.
-static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
+// Which tile a dense problem runs on: the index into the candidate table below.  blocked: the activations are in the
+// blocked layout, which the three largest tiles read (their waves then load activation fragments straight from memory).
+static int dense_choice(long M, long N, long K, bool blocked) {
     const long cus = device_cus();
-    auto tiles = [&](int bm, int bn) { return long((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
+    auto tiles = [&](int bm, int bn) { return long((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     // The tile is the one a small cost model makes fastest.  A launch runs its tiles in waves of (CUs x workgroups that
     // share a CU); a wave costs F + S per 128 of K and not less than W, all three measured per configuration and per
     // number of co-resident workgroups (four Qwen3-1.7B layer shapes and five others, K = 128 ... 6144, M = 64 ... 8192:
@@ -876,14 +911,20 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
         {64, 64, 1, {1.1f, 0, 0}, {0.26f, 0, 0}, {2.0f, 0, 0}, 0.97f, 1.0f},   // two K groups
         {64, 32, 1, {1.26f, 0, 0}, {0.14f, 0, 0}, {2.0f, 0, 0}, 0.95f, 0.97f},  // four K groups
     };
-    const float steps = float(a.K) / 128.0f;
-    int best = 4;
+    // the same tiles fed from blocked activations (fewer LDS bytes per MFMA: a shorter K step)
+    static const Cand cand_blocked[3] = {
+        {256, 256, 1, {6.5f, 0, 0}, {1.78f, 0, 0}, {8.4f, 0, 0}, 0.70f, 0.835f},
+        {256, 128, 1, {4.2f, 0, 0}, {0.85f, 0, 0}, {5.5f, 0, 0}, 0.74f, 0.78f},
+        {128, 128, 1, {1.4f, 0, 0}, {0.59f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
+    };
+    const float steps = float(K) / 128.0f;
+    int best = blocked ? 2 : 4;
     float best_t = 1e30f;
-    for (int c = 0; c < 7; ++c) {
-        const Cand& k = cand[c];
+    for (int c = 0; c < (blocked ? 3 : 7); ++c) {
+        const Cand& k = blocked ? cand_blocked[c] : cand[c];
         const long n = tiles(k.bm, k.bn);
-        if (c == 5 && (n > cus || a.K % 256)) continue;
-        if (c == 6 && (n > cus || a.K % 512)) continue;
+        if (c == 5 && (n > cus || K % 256)) continue;
+        if (c == 6 && (n > cus || K % 512)) continue;
         const long cap = cus * k.occ;
         const long full = n / cap, rest = n % cap;
         float t = float(full) * fmaxf(k.f[k.occ - 1] + steps * k.s[k.occ - 1], k.w[k.occ - 1]);
@@ -901,6 +942,18 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
         if (t < best_t * 0.98f) {   // candidates run from the largest tile down: a tie goes to the larger one
             best_t = t;
             best = c;
+        }
+    }
+    return best;
+}
+
+static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
+    const int best = dense_choice(a.M, a.N, a.K, a.blocked != 0);
+    if (a.blocked) {
+        switch (best) {
+            case 0: return launch_tile<256, 256, 64, 4, 2, 1, 2, false, false, 1, true>(a, bmode, (a.M + 255) / 256, s);
+            case 1: return launch_tile<256, 128, 128, 8, 1, 1, 2, false, false, 1, true>(a, bmode, (a.M + 255) / 256, s);
+            default: return launch_tile<128, 128, 128, 4, 2, 1, 2, false, false, 1, true>(a, bmode, (a.M + 127) / 128, s);
         }
     }
     switch (best) {
@@ -973,9 +1026,9 @@ int scmx_mm_i8_i32(const int8_t* xq, const int8_t* wq, int32_t* acc, int M, int 
     return scmx_mm_epi(xq, wq, nullptr, nullptr, nullptr, acc, SCMX_EPI_I32, M, N, K, stream);
 }
 
-int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, const uint32_t* codes,
-                 const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M, int N,
-                 int K, void* stream) {
+static int mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, const uint32_t* codes,
+                   const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M, int N,
+                   int K, bool blocked, void* stream) {
     DevFormat f;
     if (int rc = make_dev_format(fmt, &f)) return rc;
     if (int rc = check_gemm_common("mm_w4a8", M, N, K, epi, true, xq, xscale, wscale, res, out)) return rc;
@@ -992,14 +1045,46 @@ int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, 
     a.xq = xq; a.xscale = xscale; a.codes = codes; a.bcodes = bcodes; a.wscale = wscale; a.res = res; a.out = out;
     a.M = M; a.N = N; a.K = K; a.epi = epi; a.fmt = f;
     a.bc_row_bytes = K / f.block * f.bc_bits / 8;
+    a.blocked = blocked;
     launch_dense(a, packed_mode(f), (hipStream_t)stream);
     return check_launch("mm_w4a8");
 }
 
+int scmx_mm_w4a8(const scmx_format* fmt, const int8_t* xq, const float* xscale, const uint32_t* codes,
+                 const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M, int N,
+                 int K, void* stream) {
+    return mm_w4a8(fmt, xq, xscale, codes, bcodes, wscale, res, out, epi, M, N, K, false, stream);
+}
+
+int scmx_mm_w4a8_blocked(const scmx_format* fmt, const int8_t* xq, const float* xscale, const uint32_t* codes,
+                         const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M,
+                         int N, int K, void* stream) {
+    if (uintptr_t(xq) % 16) {
+        set_error("mm_w4a8_blocked: xq must be 16-byte aligned");
+        return SCMX_ERR_ARG;
+    }
+    return mm_w4a8(fmt, xq, xscale, codes, bcodes, wscale, res, out, epi, M, N, K, true, stream);
+}
+
+// The fused layer quantizes into whichever layout the GEMM's tile for the shape reads: blocked for the three largest
+// tiles, by rows otherwise.  Both layouts take (M rounded up to 32) x K bytes at most.
+static int quantize_and_multiply(const scmx_format* fmt, const uint16_t* x, int8_t* xq, float* xs, bool room_for_blocks,
+                                 const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const uint16_t* res,
+                                 void* out, int epi, int M, int N, int K, void* stream) {
+    const bool blocked = room_for_blocks && M > 0 && N > 0 && K % 128 == 0 && dense_choice(M, N, K, false) <= 2;
+    if (blocked) {
+        if (int rc = scmx_act_quant_blocked(x, xq, xs, M, (M + 31) & ~31, K, stream)) return rc;
+    } else {
+        if (int rc = scmx_act_quant(x, xq, xs, M, M, K, stream)) return rc;
+    }
+    return mm_w4a8(fmt, xq, xs, codes, bcodes, wscale, res, out, epi, M, N, K, blocked, stream);
+}
+
 size_t scmx_linear_w4a8_workspace(int M, int K) {
     if (M <= 0 || K <= 0) return 0;
-    const size_t q = (size_t(M) * size_t(K) + 255) & ~size_t(255);
-    return q + size_t(M) * sizeof(float);
+    const size_t Mp = (size_t(M) + 31) & ~size_t(31);   // whole 32-row blocks of the blocked layout
+    const size_t q = (Mp * size_t(K) + 255) & ~size_t(255);
+    return q + Mp * sizeof(float);
 }
 
 int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* codes, const uint8_t* bcodes,
@@ -1015,9 +1100,9 @@ int scmx_linear_w4a8(const scmx_format* fmt, const uint16_t* x, const uint32_t* 
         return SCMX_ERR_WORKSPACE;
     }
     int8_t* xq = reinterpret_cast<int8_t*>(workspace);
-    float* xs = reinterpret_cast<float*>(xq + ((size_t(M) * size_t(K) + 255) & ~size_t(255)));
-    if (int rc = scmx_act_quant(x, xq, xs, M, M, K, stream)) return rc;
-    return scmx_mm_w4a8(fmt, xq, xs, codes, bcodes, wscale, res, out, epi, M, N, K, stream);
+    const size_t Mp = (size_t(M) + 31) & ~size_t(31);
+    float* xs = reinterpret_cast<float*>(xq + ((Mp * size_t(K) + 255) & ~size_t(255)));
+    return quantize_and_multiply(fmt, x, xq, xs, true, codes, bcodes, wscale, res, out, epi, M, N, K, stream);
 }
 
 // ---- the dense layer for callers that cannot allocate ------------------------------------------------------------
@@ -1081,10 +1166,11 @@ int scmx_linear_w4a8_static(const scmx_format* fmt, const uint16_t* x, const uin
     if (!base) return SCMX_ERR_LAUNCH;
     int8_t* xq = reinterpret_cast<int8_t*>(base);
     float* xs = reinterpret_cast<float*>(base + STATIC_XQ_BYTES);
-    // every byte of xq[M, K] and xs[M] that the GEMM reads is written by the quantization first: nothing has to start
-    // at zero, whatever the previous call left behind
-    if (int rc = scmx_act_quant(x, xq, xs, M, M, K, stream)) return rc;
-    return scmx_mm_w4a8(fmt, xq, xs, codes, bcodes, wscale, res, out, epi, M, N, K, stream);
+    // every byte of xq and xs[M] that the GEMM reads is written by the quantization first (in the blocked layout: the
+    // whole last 32-row block, rows past M as zeros): nothing has to start at zero, whatever the previous call left behind
+    const size_t Mp = (size_t(M) + 31) & ~size_t(31);
+    const bool room = Mp * size_t(K) <= STATIC_XQ_BYTES && Mp <= size_t(STATIC_MAX_ROWS);
+    return quantize_and_multiply(fmt, x, xq, xs, room, codes, bcodes, wscale, res, out, epi, M, N, K, stream);
 }
 
 static int moe_common(const char* who, const int8_t* xq, const float* xscale, const int32_t* gather, int R,

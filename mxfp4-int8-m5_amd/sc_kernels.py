@@ -108,7 +108,13 @@ def _gemm(xq, wq, xscale, wscale, epi, res):
     if epi == 2:
         assert res is not None and tuple(res.shape) == (M, N) and res.dtype == torch.bfloat16
     r = _lib.ptr(res) if epi == 2 else None
-    if isinstance(wq, PackedWq):
+    if isinstance(xq, BlockedXq):
+        if not isinstance(wq, PackedWq):
+            raise ValueError("blocked activations multiply packed weights (unpack_i8's lazy handle)")
+        _lib.call("scmx_mm_w4a8_blocked", wq.fmt.c_struct(), _lib.ptr(xq.data), _lib.ptr(xscale), _lib.ptr(wq.codes),
+                  _lib.ptr(wq.bcodes), _lib.ptr(wscale if wscale is not None else wq.wscale), r, _lib.ptr(out), epi, M, N,
+                  K, _lib.stream())
+    elif isinstance(wq, PackedWq):
         _lib.call("scmx_mm_w4a8", wq.fmt.c_struct(), _lib.ptr(xq), _lib.ptr(xscale), _lib.ptr(wq.codes),
                   _lib.ptr(wq.bcodes), _lib.ptr(wscale if wscale is not None else wq.wscale), r, _lib.ptr(out), epi, M, N,
                   K, _lib.stream())
@@ -129,6 +135,32 @@ def mm_epi(xq, wq, xscale, wscale, epi, dtype=torch.bfloat16, res=None, deps=(),
     _check_dtype(dtype)
     assert epi in (1, 2, 3)
     return _gemm(xq, wq, xscale, wscale, epi, res)
+
+
+class BlockedXq:
+    """INT8 activations in the blocked layout (act_quant_blocked): what mm_epi / mm_i8_i32 take in place of the [Mp, K]
+    tensor when the weights are packed (PackedWq)."""
+
+    def __init__(self, data, M, K):
+        self.data, self.shape, self.dtype, self.device = data, (M, K), torch.int8, data.device
+
+    def rows(self):
+        """The [Mp, K] tensor act_quant returns (a copy)."""
+        Mp, K = self.data.numel() // self.shape[1], self.shape[1]
+        return self.data.view(Mp // 32, K // 32, 2, 32, 16).permute(0, 3, 1, 2, 4).reshape(Mp, K)
+
+
+def act_quant_blocked(x, Mp=None):
+    """act_quant for prefill-sized GEMMs on packed weights: the same codes and scales with xq in 32 x 32 blocks in the
+    order the MFMA takes them, so that the large GEMM tiles load activation fragments straight from memory
+    (scmx_act_quant_blocked / scmx_mm_w4a8_blocked).  -> (BlockedXq, xscale f32 [Mp]), Mp a multiple of 32."""
+    M, K = x.shape
+    Mp = Mp or pad_rows(M)
+    assert x.dtype == torch.bfloat16 and Mp % 32 == 0
+    xq = torch.empty(Mp * K, dtype=torch.int8, device=x.device)
+    xs = torch.empty(Mp, dtype=torch.float32, device=x.device)
+    _lib.call("scmx_act_quant_blocked", _lib.ptr(x), _lib.ptr(xq), _lib.ptr(xs), M, Mp, K, _lib.stream())
+    return BlockedXq(xq, M, K), xs
 
 
 def linear_w4a8_workspace(M, K):

@@ -56,7 +56,8 @@ def test_version_default_format_and_workspace_size(pkg):
     assert (f.block, f.bc_bits, f.n_mult) == (d.block, d.bc_bits, len(d.mult))
     assert tuple(f.code_mag) == tuple(d.code_mag) and tuple(f.mult)[:4] == tuple(d.mult)
     for m, k in ((1, 128), (2048, 2048), (77, 6144)):
-        assert lib.scmx_linear_w4a8_workspace(m, k) == (m * k + 255) // 256 * 256 + 4 * m
+        mp = (m + 31) // 32 * 32           # whole 32-row blocks of the blocked activation layout
+        assert lib.scmx_linear_w4a8_workspace(m, k) == (mp * k + 255) // 256 * 256 + 4 * mp
 
 
 def test_argument_errors_return_before_any_launch(pkg):

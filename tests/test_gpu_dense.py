@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import bf16, layout, linear
-from tests.util import FORMATS, dev, host, llm_acts, llm_weights, product_format, random_packed
+from tests.util import FORMATS, blocked_layout, dev, host, llm_acts, llm_weights, product_format, random_packed
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -190,7 +190,8 @@ def test_bad_arguments_raise(S):
         S.act_quant(torch.zeros((4, 64), dtype=torch.bfloat16))   # CPU tensor
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (37, 64, 384), (300, 1024, 512), (700, 2048, 1152), (1100, 12288, 640)])
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (37, 64, 384), (300, 1024, 512), (700, 2048, 1152), (1100, 12288, 640),
+                                   (2047, 4096, 1024)])
 def test_linear_one_call(S, m, n, k):
     """linear_w4a8 (quantization prologue + GEMM behind one C entry point): ragged row counts, few and many column
     tiles, a caller-provided workspace that ends up holding the INT8 rows and their scales."""
@@ -203,8 +204,13 @@ def test_linear_one_call(S, m, n, k):
     y = host(S.linear_w4a8(dev(bits), dev(codes), dev(bc), dev(ws), n, workspace=work))
     assert np.array_equal(y, y_ref)
     wh = host(work)
-    assert np.array_equal(wh[:m * k].view(np.int8).reshape(m, k), xq_ref)
-    off = (m * k + 255) & ~255
+    mp = (m + 31) // 32 * 32                 # the workspace is laid out for whole 32-row blocks
+    by_rows = wh[:m * k].view(np.int8).reshape(m, k)
+    padded = np.zeros((mp, k), np.int8)
+    padded[:m] = xq_ref
+    in_blocks = wh[:mp * k].view(np.int8)    # large shapes are quantized into the blocked layout
+    assert np.array_equal(by_rows, xq_ref) or np.array_equal(in_blocks, blocked_layout(padded))
+    off = (mp * k + 255) & ~255
     assert np.array_equal(wh[off:off + 4 * m].view(np.float32), xs_ref)
 
 
@@ -354,6 +360,62 @@ def test_few_tiles_two_k_groups(S, m, n, k, fmt_i):
             assert np.array_equal(host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), 3)), linear.epilogue(acc, xs, ws, 3))
     finally:
         S.set_format(product_format(layout.DEFAULT))
+
+
+@pytest.mark.parametrize("m,k", [(200, 2048), (2048, 6144), (1, 1024), (70, 160), (33, 3072), (130, 8192), (64, 96)])
+def test_act_quant_blocked(S, m, k):
+    """The blocked quantizer writes the codes of act_quant, block by block, and the same scales."""
+    rng = np.random.default_rng(m + k)
+    bits, x = llm_acts(rng, m, k)
+    if m > 3:
+        bits[3] = 0
+        x[3] = 0
+    mp = (m + 31) // 32 * 32
+    bx, xs = S.act_quant_blocked(dev(bits), mp)
+    rq, rs = linear.act_quant(x, mp)
+    assert np.array_equal(host(bx.data), blocked_layout(rq)) and np.array_equal(host(xs), rs)
+    assert np.array_equal(host(bx.rows()), rq)
+
+
+@pytest.mark.parametrize("m,n,k,fmt_i", [(2048, 4096, 2048, 0), (2048, 2048, 6144, 0), (4096, 8192, 512, 1), (300, 1000, 1280, 0),
+                                         (70, 512, 256, 5), (1, 8, 128, 0), (2049, 4100, 384, 2), (515, 3072, 1024, 1),
+                                         (8192, 2048, 256, 0)])
+def test_blocked_activations_give_the_same_gemm(S, m, n, k, fmt_i):
+    """Activations in the blocked layout (fragments loaded from memory by the large tiles, 256x256, 256x128 or 128x128 by
+    shape) against the same activations by rows: INT32 and every epilogue bit for bit, ragged M and N included; the
+    INT32 result of the smaller shapes also against the oracle directly."""
+    fmt = FORMATS[fmt_i]
+    rng = np.random.default_rng(m + n + k)
+    codes, bc, ws, q = random_packed(rng, n, k, fmt)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    xq[0] = 127
+    mp = (m + 31) // 32 * 32
+    padded = np.zeros((mp, k), np.int8)
+    padded[:m] = xq
+    xs = (np.abs(rng.standard_normal(m)) * 1e-3 + 1e-5).astype(F32)
+    res = dev(bf16.to_bits(rng.standard_normal((m, n)).astype(F32)))
+    S.set_format(product_format(fmt))
+    try:
+        wq = S.unpack_i8(dev(codes), dev(bc), n, k, lazy=True)
+        rows, blocks = dev(xq), S.BlockedXq(dev(blocked_layout(padded)), m, k)
+        acc = S.mm_i8_i32(blocks, wq)
+        assert torch.equal(acc, S.mm_i8_i32(rows, wq))
+        if m * n * k <= 300 * 1000 * 1280:
+            assert np.array_equal(host(acc), linear.int_gemm(xq, q))
+        for epi in (1, 2, 3):
+            if epi == 3 and n % 8:
+                continue
+            a = S.mm_epi(blocks, wq, dev(xs), dev(ws), epi, res=res if epi == 2 else None)
+            b = S.mm_epi(rows, wq, dev(xs), dev(ws), epi, res=res if epi == 2 else None)
+            assert torch.equal(a, b), epi
+    finally:
+        S.set_format(product_format(layout.DEFAULT))
+
+
+def test_blocked_activations_need_packed_weights(S):
+    bx, _ = S.act_quant_blocked(torch.zeros((32, 128), dtype=torch.bfloat16, device="cuda"), 32)
+    with pytest.raises(ValueError):
+        S.mm_i8_i32(bx, torch.zeros((8, 128), dtype=torch.int8, device="cuda"))
 
 
 def test_random_shapes_formats_and_epilogues(S):

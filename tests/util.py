@@ -50,6 +50,13 @@ def random_packed(rng, n, k, fmt=layout.DEFAULT):
     return codes, bc, ws, layout.decode(codes, bc, n, k, fmt)
 
 
+def blocked_layout(xq):
+    """INT8 activations [Mp, K] (Mp % 32 == 0, K % 32 == 0) -> the flat blocked layout of scmx_act_quant_blocked: 32 x 32
+    blocks, block (m / 32, k / 32) at ((m / 32) * (K / 32) + k / 32) KB, inside it row r, k half h at (32 h + r) * 16."""
+    mp, k = xq.shape
+    return np.ascontiguousarray(xq.reshape(mp // 32, 32, k // 32, 2, 16).transpose(0, 2, 3, 1, 4)).reshape(-1)
+
+
 def product_format(fmt):
     """oracle layout.Format -> the product's sc_format.Format."""
     from mxfp4_int8_m5_amd import sc_format
