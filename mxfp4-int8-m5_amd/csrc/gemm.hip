@@ -1071,9 +1071,10 @@ int scmx_mm_w4a8_blocked(const scmx_format* fmt, const int8_t* xq, const float* 
 static int quantize_and_multiply(const scmx_format* fmt, const uint16_t* x, int8_t* xq, float* xs, bool room_for_blocks,
                                  const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const uint16_t* res,
                                  void* out, int epi, int M, int N, int K, void* stream) {
-    const bool blocked = room_for_blocks && M > 0 && N > 0 && K % 128 == 0 && dense_choice(M, N, K, false) <= 2;
+    const long long Mp = (static_cast<long long>(M) + 31) & ~31LL;
+    const bool blocked = room_for_blocks && M > 0 && Mp <= (1LL << 30) && N > 0 && K % 128 == 0 && dense_choice(M, N, K, false) <= 2;
     if (blocked) {
-        if (int rc = scmx_act_quant_blocked(x, xq, xs, M, (M + 31) & ~31, K, stream)) return rc;
+        if (int rc = scmx_act_quant_blocked(x, xq, xs, M, int(Mp), K, stream)) return rc;
     } else {
         if (int rc = scmx_act_quant(x, xq, xs, M, M, K, stream)) return rc;
     }

@@ -84,7 +84,7 @@ int main() {
         ++failures;
     }
     if (scmx_linear_w4a8_workspace(2048, 2048) != size_t(2048) * 2048 + 4 * 2048 ||
-        scmx_linear_w4a8_workspace(1, 128) != 256 + 4 || scmx_linear_w4a8_workspace(0, 128) != 0 ||
+        scmx_linear_w4a8_workspace(1, 128) != 32 * 128 + 4 * 32 || scmx_linear_w4a8_workspace(0, 128) != 0 ||
         scmx_linear_w4a8_static_max_elements() != (size_t(16) << 20) || scmx_linear_w4a8_static_max_rows() != 16384) {
         printf("FAIL workspace sizes\n");
         ++failures;
@@ -109,6 +109,10 @@ int main() {
     expect(scmx_act_quant(nullptr, oq, of, 4, 4, 128, nullptr), SCMX_ERR_ARG, "act_quant null x");
     expect(scmx_act_quant(h[0], oq, of, 5, 4, 128, nullptr), SCMX_ERR_ARG, "act_quant Mp < M");
     expect(scmx_act_quant(h[0], oq, of, 4, 4, 12, nullptr), SCMX_ERR_ARG, "act_quant K % 8");
+    expect(scmx_act_quant_blocked(nullptr, oq, of, 4, 32, 128, nullptr), SCMX_ERR_ARG, "act_quant_blocked null x");
+    expect(scmx_act_quant_blocked(h[0], oq, of, 4, 4, 128, nullptr), SCMX_ERR_ARG, "act_quant_blocked Mp % 32");
+    expect(scmx_act_quant_blocked(h[0], oq, of, 40, 32, 128, nullptr), SCMX_ERR_ARG, "act_quant_blocked Mp < M");
+    expect(scmx_act_quant_blocked(h[0], oq, of, 4, 32, 48, nullptr), SCMX_ERR_ARG, "act_quant_blocked K % 32");
     expect(scmx_mm_i8_i32(xq, xq, oi[0], 4, 8, 100, nullptr), SCMX_ERR_ARG, "mm_i8_i32 K % 128");
     expect(scmx_mm_i8_i32(xq, nullptr, oi[0], 4, 8, 128, nullptr), SCMX_ERR_ARG, "mm_i8_i32 null wq");
     expect(scmx_mm_i8_i32(xq, xq, oi[0], 65536, 8, 65536, nullptr), SCMX_ERR_ARG, "mm_i8_i32 M*K beyond 32-bit offsets");
@@ -118,6 +122,9 @@ int main() {
     expect(scmx_mm_epi(xq, xq + 1, f0, f1, nullptr, out, 1, 4, 8, 128, nullptr), SCMX_ERR_ARG, "mm_epi misaligned wq");
     expect(scmx_mm_w4a8(&fmt, xq, f0, codes, bc, f1, nullptr, out, 7, 4, 8, 128, nullptr), SCMX_ERR_ARG, "mm_w4a8 unknown epilogue");
     expect(scmx_mm_w4a8(&fmt, xq, f0, codes, bc, f1, nullptr, out, 1, 4, 6, 128, nullptr), SCMX_ERR_ARG, "mm_w4a8 N % 4");
+    expect(scmx_mm_w4a8_blocked(&fmt, xq, f0, codes, bc, f1, nullptr, out, 1, 4, 6, 128, nullptr), SCMX_ERR_ARG, "mm_w4a8_blocked N % 4");
+    expect(scmx_mm_w4a8_blocked(&fmt, xq, f0, codes, bc, f1, nullptr, out, 1, 4, 8, 192, nullptr), SCMX_ERR_ARG, "mm_w4a8_blocked K % 128");
+    expect(scmx_mm_w4a8_blocked(&fmt, nullptr, f0, codes, bc, f1, nullptr, out, 1, 4, 8, 128, nullptr), SCMX_ERR_ARG, "mm_w4a8_blocked null xq");
     expect(scmx_mm_w4a8(&fmt, xq, f0, codes, nullptr, f1, nullptr, out, 1, 4, 8, 128, nullptr), SCMX_ERR_ARG, "mm_w4a8 null bcodes");
     {
         scmx_format bad = fmt;
@@ -224,10 +231,15 @@ int main() {
     expect_valid(scmx_unpack_i8(&fmt, codes, bc, oq, 4096, 2048, nullptr), "unpack_i8");
     expect_valid(scmx_act_quant(h[0], oq, of, 2048, 2048, 2048, nullptr), "act_quant");
     expect_valid(scmx_act_quant(h[0], oq, of, 7, 128, 1000, nullptr), "act_quant ragged K");
+    expect_valid(scmx_act_quant_blocked(h[0], oq, of, 2048, 2048, 2048, nullptr), "act_quant_blocked");
+    expect_valid(scmx_act_quant_blocked(h[0], oq, of, 7, 32, 96, nullptr), "act_quant_blocked short rows");
     expect_valid(scmx_mm_i8_i32(xq, xq, oi[0], 2048, 4096, 2048, nullptr), "mm_i8_i32");
     for (int epi = 0; epi <= 3; ++epi)
         expect_valid(scmx_mm_w4a8(&fmt, xq, f0, codes, bc, f1, h[0], out, epi, 2048, 12288, 2048, nullptr), "mm_w4a8");
     expect_valid(scmx_mm_w4a8(&fmt, xq, f0, codes, bc, f1, nullptr, out, 1, 1, 4, 128, nullptr), "mm_w4a8 smallest");
+    for (int epi = 0; epi <= 3; ++epi)
+        expect_valid(scmx_mm_w4a8_blocked(&fmt, xq, f0, codes, bc, f1, h[0], out, epi, 2048, 12288, 2048, nullptr), "mm_w4a8_blocked");
+    expect_valid(scmx_mm_w4a8_blocked(&fmt, xq, f0, codes, bc, f1, nullptr, out, 1, 1, 4, 128, nullptr), "mm_w4a8_blocked smallest");
     expect_valid(scmx_mm_w4a8(&fmt, xq, f0, codes, bc, f1, nullptr, out, 1, 8192, 2048, 6144, nullptr), "mm_w4a8 M = 8192");
     expect_valid(scmx_linear_w4a8(&fmt, h[0], codes, bc, f1, nullptr, out, 1, 2048, 4096, 2048, wsp,
                                   scmx_linear_w4a8_workspace(2048, 2048), nullptr),
@@ -285,11 +297,15 @@ int main() {
         }
         expect_status(scmx_unpack_i8(&f, (const uint32_t*)maybe(codes), bc, oq, r(), r(), nullptr), "fuzz unpack_i8");
         expect_status(scmx_act_quant((const uint16_t*)maybe(h[0]), oq, of, r(), r(), r(), nullptr), "fuzz act_quant");
+        expect_status(scmx_act_quant_blocked((const uint16_t*)maybe(h[0]), oq, of, r(), r(), r(), nullptr), "fuzz act_quant_blocked");
         expect_status(scmx_mm_epi(xq, (const int8_t*)maybe(xq), f0, f1, (const uint16_t*)maybe(h[0]), out, int(rng() % 6) - 1, r(), r(), r(),
                                   nullptr),
                       "fuzz mm_epi");
         expect_status(scmx_mm_w4a8(&f, xq, f0, codes, bc, f1, (const uint16_t*)maybe(h[0]), out, int(rng() % 6) - 1, r(), r(), r(), nullptr),
                       "fuzz mm_w4a8");
+        expect_status(scmx_mm_w4a8_blocked(&f, xq, f0, codes, bc, f1, (const uint16_t*)maybe(h[0]), out, int(rng() % 6) - 1, r(), r(), r(),
+                                           nullptr),
+                      "fuzz mm_w4a8_blocked");
         const int lm = r(), lk = r();
         expect_status(scmx_linear_w4a8(&f, h[0], codes, bc, f1, nullptr, out, 1, lm, r(), lk, wsp,
                                        (rng() % 2) ? scmx_linear_w4a8_workspace(lm, lk) : size_t(r()), nullptr),
