@@ -194,39 +194,46 @@ def main():
 
     # the same step without its prologues (activations quantized beforehand), and the prologues alone: where the
     # difference between `value` and the GEMM kernel's rate goes
-    pre = {}
-    for k in xs_in:
-        xq = torch.empty((M_TOKENS, k), dtype=torch.int8, device=dev)
-        xs = torch.empty(M_TOKENS, dtype=torch.float32, device=dev)
-        check(lib.scmx_act_quant(xs_in[k].data_ptr(), xq.data_ptr(), xs.data_ptr(), M_TOKENS, M_TOKENS, k, sp))
-        pre[k] = (xq, xs)
-    gcalls = [[(C.byref(fmt), pre[k][0].data_ptr(), pre[k][1].data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(),
-                None, out.data_ptr(), 1, M_TOKENS, n, k, sp) for (name, n, k), (codes, bc, ws), out in zip(LAYERS, st, outs)]
-              for st in sets]
+    # (in the layout the fused layer quantizes into for the shape: by rows, or in 32x32 blocks for the large tiles)
+    def quantized(x, m, n, k):
+        blocked = bool(lib.scmx_mm_w4a8_prefers_blocked(m, n, k))
+        mp = (m + 31) // 32 * 32
+        xq = torch.empty(mp * k, dtype=torch.int8, device=dev)
+        xs = torch.empty(mp, dtype=torch.float32, device=dev)
+        quant = lib.scmx_act_quant_blocked if blocked else lib.scmx_act_quant
+        qargs = (x.data_ptr(), xq.data_ptr(), xs.data_ptr(), m, mp if blocked else m, k, sp)
+        check(quant(*qargs))
+        return xq, xs, (lib.scmx_mm_w4a8_blocked if blocked else lib.scmx_mm_w4a8), quant, qargs, blocked
+
+    pre = [quantized(xs_in[k], M_TOKENS, n, k) for _, n, k in LAYERS]
+    gcalls = [[(pre[li][2], (C.byref(fmt), pre[li][0].data_ptr(), pre[li][1].data_ptr(), codes.data_ptr(), bc.data_ptr(),
+                             ws.data_ptr(), None, out.data_ptr(), 1, M_TOKENS, n, k, sp))
+               for li, ((name, n, k), (codes, bc, ws), out) in enumerate(zip(LAYERS, st, outs))] for st in sets]
 
     def run_gemms(i):
-        for args in gcalls[i % n_sets]:
-            check(lib.scmx_mm_w4a8(*args))
+        for mm, args in gcalls[i % n_sets]:
+            check(mm(*args))
 
     def run_prologues(i):
-        for _, _, k in LAYERS:
-            check(lib.scmx_act_quant(xs_in[k].data_ptr(), pre[k][0].data_ptr(), pre[k][1].data_ptr(), M_TOKENS, M_TOKENS,
-                                     k, sp))
+        for _, _, _, quant, qargs, _ in pre:
+            check(quant(*qargs))
     ms_gemms, _ = timeit(run_gemms, a.steps, reps=a.reps, warm_s=0.3)
     ms_pro, _ = timeit(run_prologues, a.steps, reps=a.reps, warm_s=0.2)
     step_parts = {"step_ms": round(ms_step, 4), "step_ms_min": round(ms_step_min, 4),
                   "gemms_only_ms": round(ms_gemms, 4), "gemms_only_tops": round(ops_step / ms_gemms / 1e9, 1),
                   "prologues_only_ms": round(ms_pro, 4),
                   "value_over_gemms_only": round(ms_gemms / ms_step, 3),
-                  "note": "4 layers per step; gemms_only = the four scmx_mm_w4a8 launches back to back on pre-quantized "
-                          "activations; prologues_only = the four scmx_act_quant launches"}
+                  "activation_layout": {name: "blocked" if p[5] else "rows" for (name, _, _), p in zip(LAYERS, pre)},
+                  "note": "4 layers per step; gemms_only = the four GEMM launches of the step back to back on pre-quantized "
+                          "activations (scmx_mm_w4a8_blocked where the fused layer quantizes into 32x32 blocks, else "
+                          "scmx_mm_w4a8); prologues_only = its four activation-quantization launches"}
 
     # ---- roofline of the dominant kernel (the fused-unpack GEMM alone, activations pre-quantized) -------------------
     per_shape = {}
     tot_ops = tot_ms = 0.0
     for li, (name, n, k) in enumerate(LAYERS):
         argl = [g[li] for g in gcalls]
-        ms, ms_min = timeit(lambda i: check(lib.scmx_mm_w4a8(*argl[i % n_sets])), max(20, a.steps), reps=a.reps, warm_s=0.5)
+        ms, ms_min = timeit(lambda i: check(argl[i % n_sets][0](*argl[i % n_sets][1])), max(20, a.steps), reps=a.reps, warm_s=0.5)
         ops = 2.0 * M_TOKENS * n * k
         per_shape[name] = {"us": round(ms * 1e3, 2), "us_min": round(ms_min * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
                            "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
@@ -234,7 +241,7 @@ def main():
         tot_ms += ms
     achieved = tot_ops / tot_ms / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": GEMM_TRAFFIC_BYTES, "kernel": "scmx::gemm_kernel (mm_w4a8)",
+                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": GEMM_TRAFFIC_BYTES, "kernel": "scmx::gemm_kernel (mm_w4a8 / mm_w4a8_blocked, as the fused layer launches it)",
                 "note": "INT8 ops 2MNK counted as (FL)OPs; sum over the 4 layer shapes / sum of their launch durations "
                         "(median repetition of back-to-back launches between events on the launch stream), "
                         "activations pre-quantized", "per_shape": per_shape}
@@ -260,16 +267,14 @@ def main():
         for m in (512, 8192):
             for li, (name, n, k) in enumerate(LAYERS):
                 x = up(acts(rng, m, k)).to(torch.bfloat16)
-                xq = torch.empty((m, k), dtype=torch.int8, device=dev)
-                xs = torch.empty(m, dtype=torch.float32, device=dev)
                 out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
-                check(lib.scmx_act_quant(x.data_ptr(), xq.data_ptr(), xs.data_ptr(), m, m, k, sp))
+                xq, xs, mm, _, _, _ = quantized(x, m, n, k)
                 argl = []
                 for s in sets:
                     codes, bc, ws = s[li]
                     argl.append((C.byref(fmt), xq.data_ptr(), xs.data_ptr(), codes.data_ptr(), bc.data_ptr(), ws.data_ptr(),
                                  None, out.data_ptr(), 1, m, n, k, sp))
-                ms, _ = timeit(lambda i: check(lib.scmx_mm_w4a8(*argl[i % n_sets])), 20, reps=a.reps, warm_s=0.3)
+                ms, _ = timeit(lambda i: check(mm(*argl[i % n_sets])), 20, reps=a.reps, warm_s=0.3)
                 ops = 2.0 * m * n * k
                 sweep[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
                                          "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}

@@ -111,6 +111,10 @@ int scmx_mm_w4a8_blocked(const scmx_format* fmt, const int8_t* xq, const float* 
                          const uint8_t* bcodes, const float* wscale, const uint16_t* res, void* out, int epi, int M,
                          int N, int K, void* stream);
 
+/* 1 when a dense problem of this shape runs faster from blocked activations (it is large enough for the tiles that read
+ * them), 0 when the row layout is the one to quantize into; what scmx_linear_w4a8 decides by.  No device work. */
+int scmx_mm_w4a8_prefers_blocked(int M, int N, int K);
+
 /* Whole dense W4A8 linear on a bf16 input: activation quantization prologue + scmx_mm_w4a8, one call (the activations
  * are quantized into the blocked layout when the shape runs on a tile that reads it).
  * workspace must hold scmx_linear_w4a8_workspace(M, K) bytes (the INT8 activations and their scales). */

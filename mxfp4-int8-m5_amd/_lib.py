@@ -31,6 +31,7 @@ SIGNATURES = {
     "scmx_mm_epi": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_mm_w4a8": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_mm_w4a8_blocked": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "scmx_mm_w4a8_prefers_blocked": (_I, [_I, _I, _I]),
     "scmx_linear_w4a8_workspace": (_Z, [_I, _I]),
     "scmx_linear_w4a8": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "scmx_linear_w4a8_static_max_elements": (_Z, []),

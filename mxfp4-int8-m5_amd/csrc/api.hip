@@ -244,25 +244,22 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(const uint16_t* __r
 // xq as the large dense GEMM tiles take it: blocks of 32 rows x 32 k (1 KB), block (m / 32, k / 32) at
 // ((m / 32) * (K / 32) + k / 32) KB, and inside a block the 16 bytes of row r, k half h at (32 h + r) * 16 -- the order
 // in which the 64 lanes of a wave hold a 32x32x32 MFMA operand, so that a wave fetches one block with one coalesced load.
-// One wave per row, the row in registers (NJ > 0: K = 1024 NJ, lane l owns the 16-element pieces l, l + 64, ...) or read
-// twice (NJ = 0: any K % 32 == 0); eight rows per workgroup, which between them write whole 128-byte lines.  Same codes
-// and scales as act_quant_kernel: the row maximum does not depend on the order it is taken in.
+// One wave per row, eight rows per workgroup.  NJ > 0 (K = 1024 NJ): the row stays in registers (lane l owns the
+// 16-element pieces l, l + 64, ...), and the workgroup's codes meet in LDS, piece by piece, so that they leave as whole
+// 128-byte lines (8 rows x 16 bytes are adjacent in a block).  NJ = 0 (any K % 32 == 0): the row is read twice and every
+// lane writes its own 16 bytes.  Same codes and scales as act_quant_kernel: the row maximum does not depend on the
+// order it is taken in.
 template <int NJ>
 __global__ __launch_bounds__(512) void act_quant_blocked_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
                                                                 float* __restrict__ xs, int M, int Mp, int K) {
-    const int row = blockIdx.x * 8 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (row >= Mp) return;
+    __shared__ u32x4 tile[NJ > 0 ? NJ * 64 * 8 : 1];   // [piece][row of the workgroup, rotated by piece / 2 over the banks]
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row0 = blockIdx.x * 8, row = row0 + w;   // Mp is a multiple of 32: the grid covers whole groups of 8 rows
     if (NJ > 0) K = 1024 * NJ;
     const int pieces = K / 16;
-    // piece c of the row (k = 16 c ...): k slice c / 2, half c % 2
-    int8_t* const dst = xq + (size_t(row >> 5) * size_t(K >> 5)) * 1024 + size_t(row & 31) * 16;
-    auto at = [&](int c) { return reinterpret_cast<u32x4*>(dst + size_t(c >> 1) * 1024 + (c & 1) * 512); };
-    if (row >= M) {
-        for (int c = lane; c < pieces; c += 64) *at(c) = u32x4{0u, 0u, 0u, 0u};
-        if (lane == 0) xs[row] = 0.0f;
-        return;
-    }
-    const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
+    // piece c of a row (k = 16 c ...): k slice c / 2, half c % 2
+    int8_t* const blk = xq + (size_t(row0 >> 5) * size_t(K >> 5)) * 1024;
+    auto at = [&](int c, int r) { return reinterpret_cast<u32x4*>(blk + size_t(c >> 1) * 1024 + (c & 1) * 512 + (r & 31) * 16); };
     auto amax8 = [](const u32x4& v, float m) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -282,36 +279,56 @@ __global__ __launch_bounds__(512) void act_quant_blocked_kernel(const uint16_t* 
         }
         return u32x2{o[0], o[1]};
     };
-    constexpr int NR = NJ > 0 ? NJ : 1;
-    u32x4 v[NR][2];
-    float amax = 0.0f;
-    if (NJ > 0) {
+    const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
+    if constexpr (NJ > 0) {
+        u32x4 v[NJ][2];
+        float amax = 0.0f;
+        if (row < M) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                v[j][0] = xrow[2 * (lane + 64 * j)];
+                v[j][1] = xrow[2 * (lane + 64 * j) + 1];
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) amax = amax8(v[j][1], amax8(v[j][0], amax));
+        }
+        amax = wave_max(amax);
+        const float s = __fdiv_rn(amax, 127.0f);
+        const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            v[j][0] = xrow[2 * (lane + 64 * j)];
-            v[j][1] = xrow[2 * (lane + 64 * j) + 1];
+            const int c = lane + 64 * j;
+            u32x4 o = {0u, 0u, 0u, 0u};
+            if (row < M) {
+                const u32x2 lo = codes8(v[j][0], qi), hi = codes8(v[j][1], qi);
+                o = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+            tile[c * 8 + ((w + (c >> 1)) & 7)] = o;
         }
+        if (lane == 0) xs[row] = row < M ? s : 0.0f;
+        __syncthreads();
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) amax = amax8(v[j][1], amax8(v[j][0], amax));
+        for (int j = 0; j < NJ; ++j) {   // 8 consecutive threads carry one 128-byte line: the 8 rows of a piece
+            const int idx = int(threadIdx.x) + 512 * j, c = idx >> 3, r = idx & 7;
+            *at(c, row0 + r) = tile[c * 8 + ((r + (c >> 1)) & 7)];
+        }
     } else {
+        if (row >= M) {
+            for (int c = lane; c < pieces; c += 64) *at(c, row) = u32x4{0u, 0u, 0u, 0u};
+            if (lane == 0) xs[row] = 0.0f;
+            return;
+        }
+        float amax = 0.0f;
         for (int c = lane; c < pieces; c += 64) amax = amax8(xrow[2 * c + 1], amax8(xrow[2 * c], amax));
-    }
-    amax = wave_max(amax);
-    const float s = __fdiv_rn(amax, 127.0f);
-    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
-    if (NJ > 0) {
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const u32x2 lo = codes8(v[j][0], qi), hi = codes8(v[j][1], qi);
-            *at(lane + 64 * j) = u32x4{lo[0], lo[1], hi[0], hi[1]};
-        }
-    } else {
+        amax = wave_max(amax);
+        const float s = __fdiv_rn(amax, 127.0f);
+        const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
         for (int c = lane; c < pieces; c += 64) {
             const u32x2 lo = codes8(xrow[2 * c], qi), hi = codes8(xrow[2 * c + 1], qi);
-            *at(c) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            *at(c, row) = u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
+        if (lane == 0) xs[row] = s;
     }
-    if (lane == 0) xs[row] = s;
 }
 
 // ---- rot_quant: randomized Hadamard rotation of every 32-wide block, then per-token INT8 ---------------------------
@@ -480,7 +497,7 @@ int scmx_act_quant_blocked(const uint16_t* x, int8_t* xq, float* xs, int M, int 
         return SCMX_ERR_ARG;
     }
     if (Mp == 0) return SCMX_OK;
-    const dim3 grid((unsigned(Mp) + 7u) / 8u), block(512);
+    const dim3 grid(unsigned(Mp) / 8u), block(512);
     hipStream_t st = (hipStream_t)stream;
     switch (K % 1024 ? 0 : K / 1024) {   // rows of up to 8192 elements stay in registers
         case 1: act_quant_blocked_kernel<1><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;

@@ -1066,13 +1066,17 @@ int scmx_mm_w4a8_blocked(const scmx_format* fmt, const int8_t* xq, const float* 
     return mm_w4a8(fmt, xq, xscale, codes, bcodes, wscale, res, out, epi, M, N, K, true, stream);
 }
 
+int scmx_mm_w4a8_prefers_blocked(int M, int N, int K) {
+    return M > 0 && N > 0 && K > 0 && K % 128 == 0 && dense_choice(M, N, K, false) <= 2;
+}
+
 // The fused layer quantizes into whichever layout the GEMM's tile for the shape reads: blocked for the three largest
 // tiles, by rows otherwise.  Both layouts take (M rounded up to 32) x K bytes at most.
 static int quantize_and_multiply(const scmx_format* fmt, const uint16_t* x, int8_t* xq, float* xs, bool room_for_blocks,
                                  const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const uint16_t* res,
                                  void* out, int epi, int M, int N, int K, void* stream) {
     const long long Mp = (static_cast<long long>(M) + 31) & ~31LL;
-    const bool blocked = room_for_blocks && M > 0 && Mp <= (1LL << 30) && N > 0 && K % 128 == 0 && dense_choice(M, N, K, false) <= 2;
+    const bool blocked = room_for_blocks && Mp <= (1LL << 30) && scmx_mm_w4a8_prefers_blocked(M, N, K);
     if (blocked) {
         if (int rc = scmx_act_quant_blocked(x, xq, xs, M, int(Mp), K, stream)) return rc;
     } else {
