@@ -958,9 +958,9 @@ static int dense_choice(long M, long N, long K, bool blocked) {
     };
     // the same tiles fed from blocked activations (fewer LDS bytes per MFMA: a shorter K step)
     static const Cand cand_blocked[3] = {
-        {256, 256, 1, {6.5f, 0, 0}, {1.78f, 0, 0}, {8.4f, 0, 0}, 0.70f, 0.835f},
-        {256, 128, 1, {4.2f, 0, 0}, {0.85f, 0, 0}, {5.5f, 0, 0}, 0.74f, 0.78f},
-        {128, 128, 1, {1.4f, 0, 0}, {0.59f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
+        {256, 256, 1, {6.8f, 0, 0}, {1.78f, 0, 0}, {8.4f, 0, 0}, 0.70f, 0.835f},
+        {256, 128, 1, {3.8f, 0, 0}, {0.92f, 0, 0}, {5.5f, 0, 0}, 0.74f, 0.78f},
+        {128, 128, 1, {2.8f, 0, 0}, {0.58f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
     };
     const float steps = float(K) / 128.0f;
     int best = blocked ? 2 : 4;
