@@ -144,6 +144,12 @@ int scmx_linear_w4a8_static(const scmx_format* fmt, const uint16_t* x, const uin
 int scmx_rmsnorm_quant(const uint16_t* x, const uint16_t* w, float eps, int8_t* xq, float* xs, uint16_t* xn, int M,
                        int Mp, int K, void* stream);
 
+/* scmx_rmsnorm_quant writing xq in the blocked layout of scmx_act_quant_blocked (for scmx_mm_w4a8_blocked); xn stays by
+ * rows.  Same codes and scales.  Mp % 32 == 0, K % 512 == 0, K <= 4096, 16-byte aligned operands.  The same reference
+ * function (e2e/sc_kernels.py:123-174,527-533). */
+int scmx_rmsnorm_quant_blocked(const uint16_t* x, const uint16_t* w, float eps, int8_t* xq, float* xs, uint16_t* xn, int M,
+                               int Mp, int K, void* stream);
+
 /* h = res + T(acc*xscale*wscale) written to h; then, when xq != NULL, RMSNorm(h, w, eps) + INT8.
  * Replaces res_norm_quant (e2e/sc_kernels.py:177-189,536-544) and res_epilogue (:191-197,547-551). */
 int scmx_res_norm_quant(const int32_t* acc, const float* xscale, const float* wscale, const uint16_t* res,

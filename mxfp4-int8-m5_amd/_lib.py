@@ -38,6 +38,7 @@ SIGNATURES = {
     "scmx_linear_w4a8_static_max_rows": (_I, []),
     "scmx_linear_w4a8_static": (_I, [_FMT, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "scmx_rmsnorm_quant": (_I, [_P, _P, _F, _P, _P, _P, _I, _I, _I, _P]),
+    "scmx_rmsnorm_quant_blocked": (_I, [_P, _P, _F, _P, _P, _P, _I, _I, _I, _P]),
     "scmx_res_norm_quant": (_I, [_P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _P]),
     "scmx_swiglu_quant": (_I, [_P, _P, _P, _P, _P, _I, _I, _P]),
     "scmx_qkv_headnorm": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P]),

@@ -121,22 +121,42 @@ __global__ __launch_bounds__(NT) void rmsnorm_quant_kernel(const uint16_t* __res
 // elements of lanes 2 (l % 32) and 2 (l % 32) + 1 of group 2 j + l / 32: the two four-element sums stay apart through
 // the butterfly over lane distances 16 ... 1 (= 32 ... 2 there) and are added last (= distance 1); lane l then picks
 // up the sum of group l and the second butterfly runs as it does there.
-template <int CH>
-__global__ __launch_bounds__(256) void rmsnorm_quant_wave_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                                                                 float eps, int8_t* __restrict__ xq, float* __restrict__ xs,
-                                                                 uint16_t* __restrict__ xn, int M, int Mp) {
-    constexpr int K = 512 * CH;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (row >= Mp) return;
+// BLK: xq leaves in the blocked layout of the dense GEMM (32 x 32 blocks in MFMA operand order, Mp % 32 == 0): eight
+// rows per workgroup, whose codes meet in LDS -- the 16 bytes of row r, k 16 c ... at slot c * 8 + (r + c / 2) % 8 -- and
+// are stored as whole 128-byte lines (8 rows x 16 bytes are adjacent in a block).  Same codes and scales.
+template <int CH, bool BLK = false>
+__global__ __launch_bounds__(BLK ? 512 : 256) void rmsnorm_quant_wave_kernel(const uint16_t* __restrict__ x,
+                                                                             const uint16_t* __restrict__ w, float eps,
+                                                                             int8_t* __restrict__ xq, float* __restrict__ xs,
+                                                                             uint16_t* __restrict__ xn, int M, int Mp) {
+    constexpr int K = 512 * CH, RPW = BLK ? 8 : 4;
+    __shared__ u32x2 tile[BLK ? CH * 64 * 8 : 1];
+    const int wid = threadIdx.x >> 6, row0 = blockIdx.x * RPW, row = row0 + wid, lane = threadIdx.x & 63;
+    auto gather_store = [&]() {   // BLK: after every wave's codes are in LDS
+        __syncthreads();
+        int8_t* const blk = xq + (size_t(row0 >> 5) * size_t(K >> 5)) * 1024;
+        const u32x4* t16 = reinterpret_cast<const u32x4*>(tile);
+#pragma unroll
+        for (int j = 0; j < CH / 2 + CH % 2; ++j) {   // K / 16 pieces x 8 rows of 16 bytes, 512 per pass
+            const int idx = int(threadIdx.x) + 512 * j, c = idx >> 3, r = idx & 7;
+            if (CH % 2 == 0 || c < K / 16)
+                *reinterpret_cast<u32x4*>(blk + size_t(c >> 1) * 1024 + (c & 1) * 512 + ((row0 + r) & 31) * 16) =
+                    t16[c * 8 + ((r + (c >> 1)) & 7)];
+        }
+    };
+    // piece p (8 codes) of this wave's row: half p % 2 of the 16-byte slot of chunk p / 2
+    auto slot = [&](int p) { return ((p >> 1) * 8 + ((wid + (p >> 2)) & 7)) * 2 + (p & 1); };
+    if (!BLK && row >= Mp) return;
     u32x2* qrow = reinterpret_cast<u32x2*>(xq + size_t(row) * K);
     u32x4* nrow = xn ? reinterpret_cast<u32x4*>(xn + size_t(row) * K) : nullptr;
     if (row >= M) {
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-            qrow[lane + 64 * j] = u32x2{0u, 0u};
+            if (BLK) tile[slot(lane + 64 * j)] = u32x2{0u, 0u}; else qrow[lane + 64 * j] = u32x2{0u, 0u};
             if (nrow) nrow[lane + 64 * j] = u32x4{0u, 0u, 0u, 0u};
         }
         if (lane == 0) xs[row] = 0.0f;
+        if (BLK) gather_store();
         return;
     }
     const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
@@ -196,9 +216,10 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_wave_kernel(const uint16_t*
             o[e >> 1] |= (uint32_t(q0) & 0xFFu) << (16 * (e & 1));
             o[e >> 1] |= (uint32_t(q1) & 0xFFu) << (16 * (e & 1) + 8);
         }
-        qrow[lane + 64 * j] = u32x2{o[0], o[1]};
+        if (BLK) tile[slot(lane + 64 * j)] = u32x2{o[0], o[1]}; else qrow[lane + 64 * j] = u32x2{o[0], o[1]};
     }
     if (lane == 0) xs[row] = s;
+    if (BLK) gather_store();
 }
 
 // ---- res_norm_quant / res_epilogue -----------------------------------------------------------------------------
@@ -720,6 +741,31 @@ __global__ __launch_bounds__(NT) void route_topk_kernel(const uint16_t* __restri
 using namespace scmx;
 
 extern "C" {
+
+int scmx_rmsnorm_quant_blocked(const uint16_t* x, const uint16_t* w, float eps, int8_t* xq, float* xs, uint16_t* xn, int M,
+                               int Mp, int K, void* stream) {
+    if (!x || !w || !xq || !xs || Mp < M || Mp % 32 || !row_shape_ok("rmsnorm_quant_blocked", M, K, 4096) || K % 512 ||
+        (uintptr_t(x) | uintptr_t(w) | uintptr_t(xn) | uintptr_t(xq)) % 16) {
+        if (!(x && w && xq && xs) || Mp < M || Mp % 32 || K % 512 || (uintptr_t(x) | uintptr_t(w) | uintptr_t(xn) | uintptr_t(xq)) % 16)
+            set_error("rmsnorm_quant_blocked: need M <= Mp with Mp %% 32 == 0 (Mp = %d), K %% 512 == 0 and K <= 4096 (K = %d), "
+                      "16-byte aligned operands", Mp, K);
+        return SCMX_ERR_ARG;
+    }
+    if (Mp == 0) return SCMX_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(unsigned(Mp) / 8u), block(512);
+    switch (K / 512) {
+        case 1: rmsnorm_quant_wave_kernel<1, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        case 2: rmsnorm_quant_wave_kernel<2, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        case 3: rmsnorm_quant_wave_kernel<3, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        case 4: rmsnorm_quant_wave_kernel<4, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        case 5: rmsnorm_quant_wave_kernel<5, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        case 6: rmsnorm_quant_wave_kernel<6, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        case 7: rmsnorm_quant_wave_kernel<7, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+        default: rmsnorm_quant_wave_kernel<8, true><<<grid, block, 0, st>>>(x, w, eps, xq, xs, xn, M, Mp); break;
+    }
+    return check_launch("rmsnorm_quant_blocked");
+}
 
 int scmx_rmsnorm_quant(const uint16_t* x, const uint16_t* w, float eps, int8_t* xq, float* xs, uint16_t* xn, int M,
                        int Mp, int K, void* stream) {

@@ -161,20 +161,23 @@ class FusedQwen3:
         hq, hk, d = a.num_attention_heads, a.num_key_value_heads, a.head_dim
         h, L, Mp = self._embed(ids)
         nl = len(self.layers)
-        xq, xs = S.rmsnorm_quant(h, self.layers[0][0]["input_layernorm"], self.eps, Mp)
+        # prefill-sized GEMMs on packed weights read their activations in 32x32 blocks (the quantizers write either layout)
+        blk = {g: isinstance(w.unpack(), S.PackedWq) and S.prefers_blocked(Mp, w.N, w.K) for g, w in self.layers[0][1].items()}
+        quant = lambda t, g, **kw: (S.act_quant_blocked(t, Mp) if blk[g] else S.act_quant(t, Mp, **kw))   # noqa: E731
+        xq, xs = S.rmsnorm_quant(h, self.layers[0][0]["input_layernorm"], self.eps, Mp, blocked=blk["qkv"])
         for i, (nw, ws) in enumerate(self.layers):
             y = S.mm_epi(xq, ws["qkv"].unpack(), xs, ws["qkv"].wscale, 1)
             if cache[i].offset + L > cache[i].k.shape[1]:
                 raise ValueError("KV cache is full")
             o = self._attend(cache[i], self._qkv(cache[i], L, nw, y=y), L)
-            xq, xs = S.act_quant(o, Mp)
+            xq, xs = quant(o, "o")
             h = S.mm_epi(xq, ws["o"].unpack(), xs, ws["o"].wscale, 2, res=h)
-            xq, xs = S.rmsnorm_quant(h, nw["post_attention_layernorm"], self.eps)
+            xq, xs = S.rmsnorm_quant(h, nw["post_attention_layernorm"], self.eps, blocked=blk["gu"])
             act = S.mm_epi(xq, ws["gu"].unpack(), xs, ws["gu"].wscale, 3)
-            xq, xs = S.act_quant(act, nt=512)
+            xq, xs = quant(act, "down", nt=512)
             h = S.mm_epi(xq, ws["down"].unpack(), xs, ws["down"].wscale, 2, res=h)
             if i + 1 < nl:
-                xq, xs = S.rmsnorm_quant(h, self.layers[i + 1][0]["input_layernorm"], self.eps)
+                xq, xs = S.rmsnorm_quant(h, self.layers[i + 1][0]["input_layernorm"], self.eps, blocked=blk["qkv"])
         return rms_norm(h[:L], self.norm, self.eps)
 
     def _hidden_row_epi(self, ids, cache):

@@ -160,7 +160,7 @@ def act_quant_blocked(x, Mp=None):
     xq = torch.empty(Mp * K, dtype=torch.int8, device=x.device)
     xs = torch.empty(Mp, dtype=torch.float32, device=x.device)
     _lib.call("scmx_act_quant_blocked", _lib.ptr(x), _lib.ptr(xq), _lib.ptr(xs), M, Mp, K, _lib.stream())
-    return BlockedXq(xq, M, K), xs
+    return BlockedXq(xq, Mp, K), xs   # Mp rows like act_quant's tensor: the padding rows are zeros
 
 
 def linear_w4a8_workspace(M, K):
@@ -190,26 +190,35 @@ def interleave_gate_up(F_):
     return np.stack([2 * p, 2 * p + 1, F_ + 2 * p, F_ + 2 * p + 1], 1).reshape(-1)
 
 
-def _rms(x, w, eps, Mp, want_xn):
+def _rms(x, w, eps, Mp, want_xn, blocked=False):
     M, K = x.shape
     Mp = Mp or pad_rows(M)
     assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    blocked = blocked and Mp % 32 == 0 and K % 512 == 0 and K <= 4096
     xq = torch.empty((Mp, K), dtype=torch.int8, device=x.device)
     xs = torch.empty(Mp, dtype=torch.float32, device=x.device)
     xn = torch.empty((Mp, K), dtype=torch.bfloat16, device=x.device) if want_xn else None
-    _lib.call("scmx_rmsnorm_quant", _lib.ptr(x), _lib.ptr(w), _eps(eps), _lib.ptr(xq), _lib.ptr(xs), _lib.ptr(xn), M, Mp,
-              K, _lib.stream())
+    _lib.call("scmx_rmsnorm_quant_blocked" if blocked else "scmx_rmsnorm_quant", _lib.ptr(x), _lib.ptr(w), _eps(eps),
+              _lib.ptr(xq), _lib.ptr(xs), _lib.ptr(xn), M, Mp, K, _lib.stream())
+    if blocked:
+        xq = BlockedXq(xq.reshape(-1), M, K)
     return (xq, xs, xn) if want_xn else (xq, xs)
 
 
-def rmsnorm_quant(x, w, eps, Mp=None, deps=()):
-    """x [M, K] -> (xq int8 [Mp, K], xscale f32 [Mp]) of rms_norm(x, w, eps)."""
-    return _rms(x, w, eps, Mp, False)
+def rmsnorm_quant(x, w, eps, Mp=None, deps=(), blocked=False):
+    """x [M, K] -> (xq int8 [Mp, K], xscale f32 [Mp]) of rms_norm(x, w, eps).  blocked: xq as a BlockedXq (the layout of
+    act_quant_blocked) where the shape allows it (Mp % 32 == 0, K % 512 == 0, K <= 4096), by rows otherwise."""
+    return _rms(x, w, eps, Mp, False, blocked)
 
 
-def rmsnorm_quant_n(x, w, eps, Mp=None, deps=()):
+def rmsnorm_quant_n(x, w, eps, Mp=None, deps=(), blocked=False):
     """rmsnorm_quant that also returns the normalized bf16 rows: (xq, xscale, xn [Mp, K])."""
-    return _rms(x, w, eps, Mp, True)
+    return _rms(x, w, eps, Mp, True, blocked)
+
+
+def prefers_blocked(M, N, K):
+    """Whether a dense [M, K] x [N, K]^T problem on packed weights runs faster from blocked activations."""
+    return bool(_lib.load().scmx_mm_w4a8_prefers_blocked(M, N, K))
 
 
 def res_norm_quant(acc, xscale, wscale, res, w, eps, deps=()):

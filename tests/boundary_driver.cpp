@@ -158,6 +158,9 @@ int main() {
            "linear_w4a8_static K = 0");
     expect(scmx_rmsnorm_quant(h[0], nullptr, 1e-6f, oq, of, nullptr, 4, 4, 128, nullptr), SCMX_ERR_ARG, "rmsnorm_quant null weight");
     expect(scmx_rmsnorm_quant(h[0], h[1], 1e-6f, oq, of, nullptr, 4, 4, 130, nullptr), SCMX_ERR_ARG, "rmsnorm_quant K % 8");
+    expect(scmx_rmsnorm_quant_blocked(h[0], h[1], 1e-6f, oq, of, nullptr, 4, 4, 512, nullptr), SCMX_ERR_ARG, "rmsnorm_quant_blocked Mp % 32");
+    expect(scmx_rmsnorm_quant_blocked(h[0], h[1], 1e-6f, oq, of, nullptr, 4, 32, 768, nullptr), SCMX_ERR_ARG, "rmsnorm_quant_blocked K % 512");
+    expect(scmx_rmsnorm_quant_blocked(h[0], h[1], 1e-6f, oq, of, nullptr, 4, 32, 8192, nullptr), SCMX_ERR_ARG, "rmsnorm_quant_blocked K > 4096");
     expect(scmx_res_norm_quant(nullptr, f0, f1, h[0], h[1], 1e-6f, oh[0], oq, of, 4, 128, nullptr), SCMX_ERR_ARG,
            "res_norm_quant null acc");
     expect(scmx_swiglu_quant(ci, f0, f1, nullptr, of, 4, 128, nullptr), SCMX_ERR_ARG, "swiglu_quant null xq");
@@ -246,6 +249,7 @@ int main() {
                  "linear_w4a8");
     expect_valid(scmx_linear_w4a8_static(&fmt, h[0], codes, bc, f1, nullptr, out, 1, 2048, 4096, 2048, nullptr), "linear_w4a8_static");
     expect_valid(scmx_rmsnorm_quant(h[0], h[1], 1e-6f, oq, of, oh[0], 200, 256, 2048, nullptr), "rmsnorm_quant");
+    expect_valid(scmx_rmsnorm_quant_blocked(h[0], h[1], 1e-6f, oq, of, oh[0], 200, 256, 2048, nullptr), "rmsnorm_quant_blocked");
     expect_valid(scmx_res_norm_quant(ci, f0, f1, h[0], h[1], 1e-6f, oh[0], oq, of, 256, 2048, nullptr), "res_norm_quant");
     expect_valid(scmx_swiglu_quant(ci, f0, f1, oq, of, 256, 6144, nullptr), "swiglu_quant");
     expect_valid(scmx_qkv_headnorm(nullptr, f0, f1, h[0], h[1], h[2], 1e-6f, oh[0], oh[1], oh[2], 200, 16, 8, 128, nullptr),
@@ -312,6 +316,7 @@ int main() {
                       "fuzz linear_w4a8");
         expect_status(scmx_linear_w4a8_static(&f, h[0], codes, bc, f1, nullptr, out, 1, r(), r(), r(), nullptr), "fuzz linear_w4a8_static");
         expect_status(scmx_rmsnorm_quant(h[0], h[1], 1e-6f, oq, of, (uint16_t*)maybe(oh[0]), r(), r(), r(), nullptr), "fuzz rmsnorm_quant");
+        expect_status(scmx_rmsnorm_quant_blocked(h[0], h[1], 1e-6f, oq, of, (uint16_t*)maybe(oh[0]), r(), r(), r(), nullptr), "fuzz rmsnorm_quant_blocked");
         expect_status(scmx_res_norm_quant(ci, f0, f1, h[0], h[1], 1e-6f, oh[0], (int8_t*)maybe(oq), of, r(), r(), nullptr),
                       "fuzz res_norm_quant");
         expect_status(scmx_swiglu_quant(ci, f0, f1, oq, of, r(), r(), nullptr), "fuzz swiglu_quant");

@@ -420,7 +420,7 @@ def test_blocked_activations_need_packed_weights(S):
 
 def test_random_shapes_formats_and_epilogues(S):
     """Fifty seeded random problems (ragged M and N, K of 1 to 8 K steps, every test format, every epilogue) through
-    the dense GEMM, and row 0 of each through the GEMV: bit-exact against the oracle."""
+    the dense GEMM (activations by rows and in blocks), and row 0 of each through the GEMV: bit-exact against the oracle."""
     from mxfp4_int8_m5_amd import sc_decode as G
     rng = np.random.default_rng(2024)
     done = 0
@@ -447,6 +447,15 @@ def test_random_shapes_formats_and_epilogues(S):
                 got = host(S.mm_epi(dev(xq), wq, dev(xs), dev(ws), epi, res=dev(res) if epi == 2 else None))
                 want = linear.epilogue(acc, xs, ws, epi, res if epi == 2 else None)
             assert np.array_equal(got[:m], want), (done, fmt, m, n, k, epi)
+            mp = (m + 31) // 32 * 32                      # the same problem from blocked activations
+            padded = np.zeros((mp, k), np.int8)
+            padded[:m] = xq
+            blocks = S.BlockedXq(dev(blocked_layout(padded)), m, k)
+            if epi == 0:
+                got_b = host(S.mm_i8_i32(blocks, wq))
+            else:
+                got_b = host(S.mm_epi(blocks, wq, dev(xs), dev(ws), epi, res=dev(res) if epi == 2 else None))
+            assert np.array_equal(got_b[:m], want), ("blocked", done, fmt, m, n, k, epi)
             ev = epi if epi else 1
             y = host(G.gemv(dev(xq[0]), dev(codes), dev(bc), dev(xs[:1]), dev(ws), n, ev, res=dev(res[0]) if ev == 2 else None,
                             fmt=pf))

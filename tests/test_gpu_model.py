@@ -23,17 +23,17 @@ def tiny():
     return make_tiny(4, 2, 64)
 
 
-def make_tiny(hq, hk, head_dim):
+def make_tiny(hq, hk, head_dim, hidden=256):
     from mxfp4_int8_m5_amd import fused_qwen3 as Q, sc_weights as W
-    args = Q.Qwen3Args(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=hq,
+    args = Q.Qwen3Args(hidden_size=hidden, intermediate_size=512, num_hidden_layers=2, num_attention_heads=hq,
                        num_key_value_heads=hk, head_dim=head_dim, vocab_size=320, rope_theta=1e4)
     g = torch.Generator().manual_seed(0)
     rnd = lambda *s, sc=1.0: torch.randn(*s, generator=g) * sc   # noqa: E731
     state = {"model.embed_tokens.weight": rnd(args.vocab_size, args.hidden_size),
              "model.norm.weight": 1 + rnd(args.hidden_size, sc=0.1)}
-    shapes = {"self_attn.q_proj": (hq * head_dim, 256), "self_attn.k_proj": (hk * head_dim, 256),
-              "self_attn.v_proj": (hk * head_dim, 256), "self_attn.o_proj": (256, hq * head_dim),
-              "mlp.gate_proj": (512, 256), "mlp.up_proj": (512, 256), "mlp.down_proj": (256, 512)}
+    shapes = {"self_attn.q_proj": (hq * head_dim, hidden), "self_attn.k_proj": (hk * head_dim, hidden),
+              "self_attn.v_proj": (hk * head_dim, hidden), "self_attn.o_proj": (hidden, hq * head_dim),
+              "mlp.gate_proj": (512, hidden), "mlp.up_proj": (512, hidden), "mlp.down_proj": (hidden, 512)}
     for i in range(args.num_hidden_layers):
         p = f"model.layers.{i}."
         for n in ("input_layernorm", "post_attention_layernorm"):
@@ -104,6 +104,24 @@ def test_prefill_against_float_model(tiny, epilogue):
     ref = float_model(Q, args, state, packed, ids)
     assert h.shape == ref.shape
     assert rel(h, ref) < 3e-2, rel(h, ref)       # two blocks of INT8 activations + bf16 residual stream
+
+
+def test_prefill_from_blocked_activations_gives_the_same_bits(monkeypatch):
+    """Prefill-sized GEMMs read their activations in 32x32 blocks (every quantizer of the block writes that layout); with
+    the choice forced on for a small model the hidden states equal those of the row layout bit for bit."""
+    Q, args, state, packed = make_tiny(4, 2, 64, hidden=512)
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    ids = torch.randint(0, args.vocab_size, (150,), generator=torch.Generator().manual_seed(5)).cuda()
+    m = Q.FusedQwen3(args, state, packed)
+    by_rows = m.hidden(ids)
+    seen = []
+    real = S.act_quant_blocked
+    monkeypatch.setattr(S, "prefers_blocked", lambda M, N, K: True)
+    monkeypatch.setattr(S, "act_quant_blocked", lambda *a, **k: (seen.append(1), real(*a, **k))[1])
+    in_blocks = m.hidden(ids)
+    assert len(seen) == 2 * args.num_hidden_layers          # the o_proj and down inputs of every block
+    assert torch.equal(in_blocks, by_rows)
+    assert rel(by_rows, float_model(Q, args, state, packed, ids.cpu())) < 3e-2
 
 
 def test_prefill_with_this_librarys_attention_kernel():

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import bf16, layout, linear
-from tests.util import dev, host, llm_acts
+from tests.util import blocked_layout, dev, host, llm_acts
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -35,6 +35,14 @@ def test_rmsnorm_quant(S, m, k):
     xf, wf = bf16.from_bits(x).astype(np.float64), bf16.from_bits(nw).astype(np.float64)
     ref = wf * xf / np.sqrt((xf ** 2).mean(1, keepdims=True) + 1e-6)
     assert linear.rel_fro(bf16.from_bits(host(xn))[:m], ref) < 1e-2
+    # the same codes block by block (the layout the large dense GEMM tiles read), where the shape allows it
+    bq, bs, bn = S.rmsnorm_quant_n(dev(x), dev(nw), 1e-6, blocked=True)
+    if k % 512 == 0 and k <= 4096:
+        assert isinstance(bq, S.BlockedXq) and np.array_equal(host(bq.data), blocked_layout(rq))
+        assert np.array_equal(host(bq.rows()), rq)
+    else:
+        assert np.array_equal(host(bq), rq)
+    assert np.array_equal(host(bs), rs) and np.array_equal(host(bn), rn)
 
 
 def test_res_norm_quant_and_res_epilogue(S):
