@@ -55,10 +55,10 @@ enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3,
 // K / KG of the reduction out of LDS stages of its own, and the INT32 partial sums meet in LDS before the epilogue (exact:
 // integer addition is associative).  A CU then runs KG times the waves on the same tile count.
 template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false,
-          int KG = 1, bool AD = false, int KS = 1>
-__global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const GemmArgs a) {
+          int KG = 1, bool AD = false>
+__global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const GemmArgs a) {
     constexpr int NSTAGE = 3;   // LDS stages: one being read, one ready, one being written
-    constexpr int NT = WGM * WGN * KS * 64;   // threads of one K group
+    constexpr int NT = WGM * WGN * 64;   // threads of one K group
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int MI = WTM / 32, NI = WTN / 32;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && (BK == 64 || BK == 128), "tile must be whole 32x32x32 MFMAs");
@@ -86,24 +86,14 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     constexpr int EPI_BYTES = WGM * WGN * WTM * (WTN * 2 + 16);
     static_assert(KG == 1 || (!PK && !SKIP), "K groups: staged dense tiles");
     static_assert(!AD || (!PK && !SKIP && KG == 1), "activation fragments from memory: staged dense tiles");
-    // KS = 2 (with AD): two sets of WGM x WGN waves share the tile AND its LDS stages; set s multiplies k slices
-    // s * NKK / 2 ... of every K step.  A wave tile is then twice as tall for the same eight waves -- half the weight
-    // fragment reads per MFMA -- and the two sets swap halves of their INT32 sums through LDS before the epilogue (exact),
-    // each finishing the 32-row blocks it keeps.
-    static_assert(KS == 1 || (KS == 2 && AD && MI % 2 == 0 && BK == 128), "k-slice sets: two, on tiles fed from blocked activations");
-    constexpr int EMI = MI / KS, EWTM = WTM / KS;   // what a wave carries through the epilogue
     constexpr int GROUP_BYTES = NSTAGE * STAGE;
     // after the K loop: group 0's output tiles (the widest epilogue's) from 0, then the other groups' partial sums
     constexpr int PART_BYTES = NT * MI * NI * 64;
     constexpr int PART_BASE = WGM * WGN * WTM * (WTN * 4 + 16);
     constexpr int KG_BYTES = PART_BASE + (KG - 1) * PART_BYTES > KG * GROUP_BYTES ? PART_BASE + (KG - 1) * PART_BYTES : KG * GROUP_BYTES;
     static_assert(KG == 1 || KG_BYTES <= 160 * 1024, "stages and partial sums fit the CU's LDS");
-    constexpr int XCH_BYTES = KS > 1 ? NT * EMI * NI * 64 : 0;   // the halves the two k-slice sets swap
-    static_assert(XCH_BYTES <= 150 * 1024, "the swapped halves fit the CU's LDS");
-    constexpr int SMEM_BYTES = KS > 1   ? (XCH_BYTES > NSTAGE * STAGE ? XCH_BYTES : NSTAGE * STAGE)
-                               : KG > 1 ? KG_BYTES
-                               : (EPI_BYTES > NSTAGE * STAGE && EPI_BYTES <= 150 * 1024) ? EPI_BYTES
-                                                                                          : NSTAGE * STAGE;
+    constexpr int SMEM_BYTES =
+        KG > 1 ? KG_BYTES : (EPI_BYTES > NSTAGE * STAGE && EPI_BYTES <= 150 * 1024) ? EPI_BYTES : NSTAGE * STAGE;
     __shared__ __attribute__((aligned(16))) int8_t smem[SMEM_BYTES];
     // scales of the tile's rows and columns, fetched before the K loop so that the epilogue does not start with a
     // round trip to memory
@@ -115,9 +105,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     const int kg = KG == 1 ? 0 : __builtin_amdgcn_readfirstlane(int(threadIdx.x) / NT);   // K group (wave-uniform)
     const int tid = KG == 1 ? int(threadIdx.x) : int(threadIdx.x) % NT, lane = tid & 63, wave = tid >> 6;
     int8_t* const sm = smem + kg * GROUP_BYTES;   // this group's stages
-    const int ks = KS == 1 ? 0 : __builtin_amdgcn_readfirstlane(wave / (WGM * WGN));   // k-slice set (wave-uniform)
-    const int wv = KS == 1 ? wave : wave % (WGM * WGN);
-    const int wm = SKIP ? wv / WGN : wv % WGM, wn = SKIP ? wv % WGN : wv / WGM;
+    const int wm = SKIP ? wave / WGN : wave % WGM, wn = SKIP ? wave % WGN : wave / WGM;
 
     // ---- which tile ------------------------------------------------------------------------------------------
     const int num_n = (a.N + BN - 1) / BN;
@@ -356,10 +344,9 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     // origins are multiples of 32 rows, so the swizzle term depends on the lane only
     const int lr = lane & 31, half = lane >> 5;
     const int sw = (lr / RPB) & (CPR - 1);
-    constexpr int NKL = NKK / KS;   // k slices of a step that this wave multiplies: ks * NKL ...
-    int koff[NKL];
+    int koff[NKK];
 #pragma unroll
-    for (int kk = 0; kk < NKL; ++kk) koff[kk] = ((2 * (ks * NKL + kk) + half) ^ sw) << 4;
+    for (int kk = 0; kk < NKK; ++kk) koff[kk] = ((2 * kk + half) ^ sw) << 4;
     const int a_frag = (wm * WTM + lr) * BK;
     const int b_frag = A_BYTES + (wn * WTN + lr) * BK;
 
@@ -503,7 +490,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     // Fragments are fetched FD - 1 k slices ahead of the MFMAs that use them, into FD rotating register buffers; the
     // slices fetched at the end of an iteration belong to the next step's stage.
     constexpr int AHEAD = FD - 1;
-    static_assert(AHEAD >= 1 && AHEAD <= NKL, "fragment prefetch distance");
+    static_assert(AHEAD >= 1 && AHEAD <= NKK, "fragment prefetch distance");
     [[maybe_unused]] v4i fa[FD][MI], fb[FD][NI];
     auto load_frags = [&](const int8_t* src, int kk, v4i (&xa)[MI], v4i (&xb)[NI]) {
         if (SKIP && mi_active == 0) return;
@@ -517,18 +504,18 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     // k half l / 32, 16 bytes each), block (m / 32, k / 32) at ((m / 32) * (K / 32) + k / 32) KB.  Every wave loads the
     // fragments of its own rows straight into registers, two K steps ahead, in three buffers that rotate with the LDS
     // stages: the activation tile never passes through LDS.
-    [[maybe_unused]] v4i fad[NSTAGE][NKL][MI];
+    [[maybe_unused]] v4i fad[NSTAGE][NKK][MI];
     [[maybe_unused]] int ad_src[MI];
     if constexpr (AD) {
         const int last_block = (a.M + 31) / 32 - 1;
 #pragma unroll
         for (int i = 0; i < MI; ++i)
             ad_src[i] = int(uint32_t(min((m0 + wm * WTM) / 32 + i, last_block)) * uint32_t(K >> 5) * 1024u + uint32_t(lane) * 16u +
-                            uint32_t(kbase) * 32u + uint32_t(ks * NKL) * 1024u);
+                            uint32_t(kbase) * 32u);
     }
     auto load_ad = [&](int buf, int k0) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kk = 0; kk < NKL; ++kk)
+        for (int kk = 0; kk < NKK; ++kk)
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, ad_src[i] + kk * 1024, k0 * 32, 0);
@@ -557,7 +544,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
         constexpr bool ST = decltype(stage_tag)::value;      // false in the last two steps: nothing left to stage
         constexpr int wr = (rd + 2) % NSTAGE;                // stage of step kt + 2
         constexpr int nx = (rd + 1) % NSTAGE;                // stage of step kt + 1
-        constexpr int ph = (NKL * rd) % FD;                  // fragment buffer of slice 0 of this step (FD divides 6 * NKL)
+        constexpr int ph = (NKK * rd) % FD;                  // fragment buffer of slice 0 of this step (FD divides 6 * NKK)
         __syncthreads();
         const int8_t* src = sm + rd * STAGE;
         const int8_t* nxt = sm + nx * STAGE;
@@ -567,11 +554,11 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
         uint32_t o[B_PER][8];
         if constexpr (AD && ST) load_ad(wr, k2);
 #pragma unroll
-        for (int kk = 0; kk < NKL; ++kk) {
-            if (kk + AHEAD < NKL)
+        for (int kk = 0; kk < NKK; ++kk) {
+            if (kk + AHEAD < NKK)
                 load_frags(src, kk + AHEAD, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
             else
-                load_frags(nxt, kk + AHEAD - NKL, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
+                load_frags(nxt, kk + AHEAD - NKK, fa[(ph + kk + AHEAD) % FD], fb[(ph + kk + AHEAD) % FD]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
@@ -581,10 +568,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[(ph + kk) % FD][j], AD ? fad[rd][kk][i] : fa[(ph + kk) % FD][i],
                                                                       acc[i][j], 0, 0, 0);
             }
-            if constexpr (ST) {
-#pragma unroll
-                for (int q = 0; q < KS; ++q) stage_slice(r, dst, k2, kk * KS + q, o);
-            }
+            if constexpr (ST) stage_slice(r, dst, k2, kk, o);
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (ST) load_global(r, k4);
@@ -709,35 +693,6 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
                     for (int r = 0; r < 16; ++r) acc[i][j][r] += other[((i * NI + j) * 16 + r) * NT + tid];
         }
     }
-    // KS = 2: a wave keeps the 32-row blocks ks * EMI ... of its tile and hands the others to its partner in the other set
-    v16i fin[KS > 1 ? EMI : 1][KS > 1 ? NI : 1];
-    if constexpr (KS > 1) {
-        v4i* xch = reinterpret_cast<v4i*>(smem);   // four registers of a thread at 16-byte word (register group) * NT + thread
-#pragma unroll
-        for (int i = 0; i < EMI; ++i)
-#pragma unroll
-            for (int j = 0; j < NI; ++j)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const v16i& give = ks ? acc[i][j] : acc[EMI + i][j];
-                    xch[((i * NI + j) * 4 + g) * NT + tid] = v4i{give[4 * g], give[4 * g + 1], give[4 * g + 2], give[4 * g + 3]};
-                }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < EMI; ++i)
-#pragma unroll
-            for (int j = 0; j < NI; ++j)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const v16i& keep = ks ? acc[EMI + i][j] : acc[i][j];
-                    const v4i got = xch[((i * NI + j) * 4 + g) * NT + (tid ^ (NT / 2))];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) fin[i][j][4 * g + r] = keep[4 * g + r] + got[r];
-                }
-        __syncthreads();   // the buffer becomes the waves' output tiles
-    }
-    auto& eacc = [&]() -> auto& { if constexpr (KS > 1) return fin; else return acc; }();
-    const int frow = wm * WTM + ks * EWTM;   // first row, inside the tile, of what this wave finishes
     auto epilogue = [&](auto epi_tag) {
     constexpr int epi = decltype(epi_tag)::value;
     constexpr int esize = epi == SCMX_EPI_I32 ? 4 : 2;
@@ -746,16 +701,16 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     constexpr int rowb = ocols * esize;                                // bytes per tile row
     constexpr int rsb = rowb + 16;                                     // padded LDS row stride
     constexpr bool fits = WGM * WGN * WTM * rsb <= SMEM_BYTES;   // per-wave tiles reuse the staging LDS
-    int8_t* wtile = smem + (fits ? wave * (EWTM * rsb) : 0);
-    const int wm0 = m0 + frow, wn0 = n0 + wn * WTN;            // wave tile origin (input column index)
+    int8_t* wtile = smem + (fits ? wave * (WTM * rsb) : 0);
+    const int wm0 = m0 + wm * WTM, wn0 = n0 + wn * WTN;            // wave tile origin (input column index)
     const bool wide = fits && (size_t(on) * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 &&
                       (epi != SCMX_EPI_RES || reinterpret_cast<uintptr_t>(a.res) % 16 == 0);
 
-    float xsv[EMI];
+    float xsv[MI];
     f32x4 wsv[NI][4];
     if (epi != SCMX_EPI_I32) {
 #pragma unroll
-        for (int i = 0; i < EMI; ++i) xsv[i] = s_xs[frow + i * 32 + lr];
+        for (int i = 0; i < MI; ++i) xsv[i] = s_xs[wm * WTM + i * 32 + lr];
 #pragma unroll
         for (int j = 0; j < NI; ++j)
 #pragma unroll
@@ -765,7 +720,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     auto emit = [&](auto wide_tag) __attribute__((always_inline)) {
     constexpr bool W = decltype(wide_tag)::value;
 #pragma unroll
-    for (int i = 0; i < EMI; ++i) {
+    for (int i = 0; i < MI; ++i) {
         const int row = i * 32 + lr;
         const int m = wm0 + row;
         const float xs = epi != SCMX_EPI_I32 ? xsv[i] : 0.0f;
@@ -776,7 +731,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
                 const int col = j * 32 + 8 * g + 4 * half;
                 const int n = wn0 + col;
                 if (epi == SCMX_EPI_I32) {
-                    const v4i v = v4i{eacc[i][j][4 * g], eacc[i][j][4 * g + 1], eacc[i][j][4 * g + 2], eacc[i][j][4 * g + 3]};
+                    const v4i v = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
                     if (W)
                         *reinterpret_cast<v4i*>(wtile + row * rsb + col * 4) = v;
                     else if (m < row_end && n < N)
@@ -787,7 +742,7 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
                 float y[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    y[r] = __fmul_rn(__fmul_rn(float(eacc[i][j][4 * g + r]), xs), w4[r]);
+                    y[r] = __fmul_rn(__fmul_rn(float(acc[i][j][4 * g + r]), xs), w4[r]);
                 uint16_t* out = reinterpret_cast<uint16_t*>(a.out);
                 if (epi == SCMX_EPI_SWIGLU) {   // (g, g, u, u) -> two outputs
                     const uint16_t s0 = swiglu_lut(a.silu, y[0], round_bf16(y[2]));
@@ -830,10 +785,10 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
     const int ocol0 = epi == SCMX_EPI_SWIGLU ? wn0 / 2 : wn0;
     // In batches of eight pieces per lane: all LDS reads (and residual loads) of a batch are in flight before the first
     // is used, instead of one round trip per piece.
-    constexpr int NP = EWTM * ppr / 64, NB = NP < 8 ? NP : 8;
-    static_assert(EWTM * ppr % 64 == 0 && NP % NB == 0, "whole batches of pieces per lane");
+    constexpr int NP = WTM * ppr / 64, NB = NP < 8 ? NP : 8;
+    static_assert(WTM * ppr % 64 == 0 && NP % NB == 0, "whole batches of pieces per lane");
 #pragma unroll 1
-    for (int p0 = lane; p0 < EWTM * ppr; p0 += 64 * NB) {
+    for (int p0 = lane; p0 < WTM * ppr; p0 += 64 * NB) {
         u32x4 v[NB], rr[NB];
         bool ok[NB], full[NB];
         int8_t* dst[NB];
@@ -890,13 +845,13 @@ __global__ __launch_bounds__(WGM* WGN* KG* KS * 64, OCC) void gemm_kernel(const 
 // ---- host dispatch ---------------------------------------------------------------------------------------------
 
 template <int BM, int BN, int BK, int WGM, int WGN, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false, int KG = 1,
-          bool AD = false, int KS = 1>
+          bool AD = false>
 static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStream_t s) {
     GemmArgs a = a_in;
     if (a.epi == SCMX_EPI_SWIGLU) a.silu = silu_table_device();
     const int num_n = (a.N + BN - 1) / BN;
     if (a.tstart) row_tiles = (row_tiles + 7) & ~7;   // grouped: whole chunks of 8 row-tile slots (spare slots exit at once)
-    const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * KG * KS * 64);
+    const dim3 grid(unsigned(row_tiles) * unsigned(num_n)), block(WGM * WGN * KG * 64);
     if constexpr (PK) {   // callers choose this tile for the two FP4-conversion formats only
         if (bmode == B_PACKED_DEFAULT)
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
@@ -904,17 +859,17 @@ static void launch_tile(const GemmArgs& a_in, int bmode, int row_tiles, hipStrea
             gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, true><<<grid, block, 0, s>>>(a);
     } else {
         if (bmode == B_INT8)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP, false, KG, AD, KS><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_INT8, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_DEFAULT)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, false, KG, AD, KS><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_DEFAULT, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, false, KG, AD, KS><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_B16M)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP, false, KG, AD, KS><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_B16M, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else if (bmode == B_PACKED_E8M0)
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP, false, KG, AD, KS><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_E8M0, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
         else
-            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP, false, KG, AD, KS><<<grid, block, 0, s>>>(a);
+            gemm_kernel<BM, BN, BK, WGM, WGN, B_PACKED_GENERIC, OCC, FD, SKIP, false, KG, AD><<<grid, block, 0, s>>>(a);
     }
 }
 
@@ -928,7 +883,7 @@ static int packed_mode(const DevFormat& f) {
 
 // Dense: one launch, with the tile a cost model of the candidates below makes fastest.
 // Which tile a dense problem runs on: the index into the candidate table below.  blocked: the activations are in the
-// blocked layout, which the three largest tiles read (their waves then load activation fragments straight from memory).
+// blocked layout, which four tiles read (their waves then load activation fragments straight from memory).
 static int dense_choice(long M, long N, long K, bool blocked) {
     const long cus = device_cus();
     auto tiles = [&](int bm, int bn) { return long((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -957,15 +912,18 @@ static int dense_choice(long M, long N, long K, bool blocked) {
         {64, 32, 1, {1.26f, 0, 0}, {0.14f, 0, 0}, {2.0f, 0, 0}, 0.95f, 0.97f},  // four K groups
     };
     // the same tiles fed from blocked activations (fewer LDS bytes per MFMA: a shorter K step)
-    static const Cand cand_blocked[3] = {
+    static const Cand cand_blocked[4] = {
         {256, 256, 1, {6.8f, 0, 0}, {1.78f, 0, 0}, {8.4f, 0, 0}, 0.70f, 0.835f},
         {256, 128, 1, {3.8f, 0, 0}, {0.92f, 0, 0}, {5.5f, 0, 0}, 0.74f, 0.78f},
         {128, 128, 1, {2.8f, 0, 0}, {0.58f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
+        // eight waves stacked along M on 64 columns: half the weight staging of the 128x128 tile per MFMA, no activation
+        // row fetched twice (2048-wide layers at M = 1024 ... 2048: 13.7 -> 12.2 us, K = 6144: 30.8 -> 28.9)
+        {256, 64, 1, {2.2f, 0, 0}, {0.55f, 0, 0}, {3.0f, 0, 0}, 0.86f, 0.97f},
     };
     const float steps = float(K) / 128.0f;
     int best = blocked ? 2 : 4;
     float best_t = 1e30f;
-    for (int c = 0; c < (blocked ? 3 : 7); ++c) {
+    for (int c = 0; c < (blocked ? 4 : 7); ++c) {
         const Cand& k = blocked ? cand_blocked[c] : cand[c];
         const long n = tiles(k.bm, k.bn);
         if (c == 5 && (n > cus || K % 256)) continue;
@@ -998,12 +956,8 @@ static void launch_dense(const GemmArgs& a, int bmode, hipStream_t s) {
         switch (best) {
             case 0: return launch_tile<256, 256, 64, 4, 2, 1, 2, false, false, 1, true>(a, bmode, (a.M + 255) / 256, s);
             case 1: return launch_tile<256, 128, 128, 8, 1, 1, 2, false, false, 1, true>(a, bmode, (a.M + 255) / 256, s);
-            default:
-                // long reductions: two k-slice sets of 2 x 2 waves (64x64 wave tiles: half the weight fragment reads per
-                // MFMA) repay the exchange of partial sums that ends them (K = 6144: 32.9 -> 31.0 us at M = 2048)
-                if (a.K >= 4096)
-                    return launch_tile<128, 128, 128, 2, 2, 1, 2, false, false, 1, true, 2>(a, bmode, (a.M + 127) / 128, s);
-                return launch_tile<128, 128, 128, 4, 2, 1, 2, false, false, 1, true>(a, bmode, (a.M + 127) / 128, s);
+            case 3: return launch_tile<256, 64, 128, 8, 1, 1, 2, false, false, 1, true>(a, bmode, (a.M + 255) / 256, s);
+            default: return launch_tile<128, 128, 128, 4, 2, 1, 2, false, false, 1, true>(a, bmode, (a.M + 127) / 128, s);
         }
     }
     switch (best) {

@@ -379,10 +379,11 @@ def test_act_quant_blocked(S, m, k):
 
 @pytest.mark.parametrize("m,n,k,fmt_i", [(2048, 4096, 2048, 0), (2048, 2048, 6144, 0), (4096, 8192, 512, 1), (300, 1000, 1280, 0),
                                          (70, 512, 256, 5), (1, 8, 128, 0), (2049, 4100, 384, 2), (515, 3072, 1024, 1),
-                                         (8192, 2048, 256, 0), (515, 1000, 4096, 1), (130, 2048, 8192, 3)])
+                                         (8192, 2048, 256, 0), (515, 1000, 4096, 1), (130, 2048, 8192, 3), (1024, 4096, 2048, 0),
+                                         (100, 128, 512, 0), (128, 32768, 256, 0)])
 def test_blocked_activations_give_the_same_gemm(S, m, n, k, fmt_i):
-    """Activations in the blocked layout (fragments loaded from memory by the large tiles, 256x256, 256x128 or 128x128 by
-    shape, the last with two k-slice sets of waves from K = 4096 on) against the same activations by rows: INT32 and every epilogue bit for bit, ragged M and N included; the
+    """Activations in the blocked layout (fragments loaded from memory by the large tiles: 256x256, 256x128, 128x128 or
+    256x64 by shape) against the same activations by rows: INT32 and every epilogue bit for bit, ragged M and N included; the
     INT32 result of the smaller shapes also against the oracle directly."""
     fmt = FORMATS[fmt_i]
     rng = np.random.default_rng(m + n + k)
