@@ -30,8 +30,8 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0        # MI355X dense INT8 MFMA, published
 # HBM-side bytes per GEMM launch (mean over the four layer launches of one step), from rocprofv3 TCC counters of this
 # workload: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, both factors calibrated on a 256 MiB device copy.  Per layer
-# (fetched + written MiB): qkv 24.5 + 16, o_proj 16.4 + 8, gate_up 41.6 + 48.4, down 48.6 + 8.
-GEMM_TRAFFIC_BYTES = int((24.5 + 16 + 16.4 + 8 + 41.6 + 48.4 + 48.6 + 8) * 2 ** 20 / 4)
+# (fetched + written MiB): qkv 24.5 + 16.1, gate_up 41.6 + 48.4, o_proj and down together 80.8 + 16.
+GEMM_TRAFFIC_BYTES = int((24.5 + 16.1 + 41.6 + 48.4 + 80.8 + 16) * 2 ** 20 / 4)
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E, published
 M_TOKENS = 2048
 LAYERS = [("qkv", 4096, 2048), ("o_proj", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]

@@ -1074,8 +1074,8 @@ int scmx_mm_w4a8_prefers_blocked(int M, int N, int K) {
     return M > 0 && N > 0 && K > 0 && K % 128 == 0 && dense_choice(M, N, K, false) <= 2;
 }
 
-// The fused layer quantizes into whichever layout the GEMM's tile for the shape reads: blocked for the three largest
-// tiles, by rows otherwise.  Both layouts take (M rounded up to 32) x K bytes at most.
+// The fused layer quantizes into whichever layout suits the shape: blocked where the row-layout model would run one of its
+// three largest tiles (the blocked tiles then win), by rows otherwise.  Both layouts take (M rounded up to 32) x K bytes at most.
 static int quantize_and_multiply(const scmx_format* fmt, const uint16_t* x, int8_t* xq, float* xs, bool room_for_blocks,
                                  const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const uint16_t* res,
                                  void* out, int epi, int M, int N, int K, void* stream) {
