@@ -54,6 +54,9 @@ enum { B_INT8 = 0, B_PACKED_DEFAULT = 1, B_PACKED_GENERIC = 2, B_PACKED_B16 = 3,
 // KG > 1 (small problems: fewer tiles than CUs): KG groups of WGM x WGN waves share the tile, each multiplies its own
 // K / KG of the reduction out of LDS stages of its own, and the INT32 partial sums meet in LDS before the epilogue (exact:
 // integer addition is associative).  A CU then runs KG times the waves on the same tile count.
+// AD (dense, activations in the blocked layout): the activation tile does not pass through LDS; every wave loads the
+// fragments of its own rows from memory, one coalesced 1 KB load per 32-row x 32-k block, two K steps ahead.  Waves must
+// then not share rows (WGN = 1, or few column groups), and only the weight rows of a stage exist in LDS.
 template <int BM, int BN, int BK, int WGM, int WGN, int BMODE, int OCC = 1, int FD = 2, bool SKIP = false, bool PK = false,
           int KG = 1, bool AD = false>
 __global__ __launch_bounds__(WGM* WGN* KG * 64, OCC) void gemm_kernel(const GemmArgs a) {
