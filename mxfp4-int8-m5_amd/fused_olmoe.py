@@ -178,8 +178,10 @@ class FusedOlmoe:
             y = S.mm_epi(xq, ws["qkv"].unpack(), xs, ws["qkv"].wscale, 1)
             q, k, v = S.qkv_fullnorm_y(y, nw["self_attn.q_norm"], nw["self_attn.k_norm"], self.eps, L, H, d)
             o = self._attention(cache[i], q, k, v, L)
-            xq, xs = S.act_quant(o, Mp)
-            h = S.mm_epi(xq, ws["o"].unpack(), xs, ws["o"].wscale, 2, res=h)
+            wo = ws["o"].unpack()   # a prefill-sized GEMM on packed weights reads its activations in 32x32 blocks
+            blocked = isinstance(wo, S.PackedWq) and S.prefers_blocked(Mp, ws["o"].N, ws["o"].K)
+            xq, xs = S.act_quant_blocked(o, Mp) if blocked else S.act_quant(o, Mp)
+            h = S.mm_epi(xq, wo, xs, ws["o"].wscale, 2, res=h)
             xq, xs, xn = S.rmsnorm_quant_n(h, nw["post_attention_layernorm"], self.eps)
             inds, scores = self.route(nw, xn, L)
             if self.record is not None:

@@ -593,6 +593,21 @@ def test_olmoe_prefill_against_float_model(tiny_moe, kw):
     assert rel(h, ref) < 4e-2, rel(h, ref)
 
 
+def test_olmoe_prefill_from_blocked_activations_gives_the_same_bits(tiny_moe, monkeypatch):
+    """The attention output projection of a long prompt reads blocked activations; forced on for the small model, the
+    hidden states are those of the row layout bit for bit."""
+    from mxfp4_int8_m5_amd import sc_kernels as S
+    O, args, state, packed = tiny_moe
+    ids = torch.randint(0, args.vocab_size, (90,), generator=torch.Generator().manual_seed(14)).cuda()
+    m = O.FusedOlmoe(args, state, packed, tile=64)
+    by_rows = m.hidden(ids)
+    seen = []
+    real = S.act_quant_blocked
+    monkeypatch.setattr(S, "prefers_blocked", lambda M, N, K: True)
+    monkeypatch.setattr(S, "act_quant_blocked", lambda *a, **k: (seen.append(1), real(*a, **k))[1])
+    assert torch.equal(m.hidden(ids), by_rows) and len(seen) == args.num_hidden_layers
+
+
 def test_olmoe_prefill_with_head_dim_128():
     """Two heads of 128: the prefill attention runs through scmx_attn_prefill (q copied to token-major first)."""
     O, args, state, packed = make_tiny_moe(2)
