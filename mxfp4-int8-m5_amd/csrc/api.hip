@@ -197,17 +197,39 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 
 // The same with the row held in registers: one wave per row, lane l owns the 16-byte pieces l, l + 64, ... (CH of
 // them, K = 512 * CH), so the row is read once and the only reduction is inside the wave.  Four rows per workgroup.
-template <int CH>
-__global__ __launch_bounds__(256) void act_quant_wave_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
-                                                             float* __restrict__ xs, int M, int Mp) {
-    constexpr int K = 512 * CH;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (row >= Mp) return;
+// BLK: xq leaves in the blocked layout of the dense GEMM's large tiles (32 x 32 blocks in MFMA operand order, described at
+// act_quant_blocked_kernel below; Mp % 32 == 0): eight rows per workgroup, whose codes meet in LDS -- the 16 bytes of row
+// r, k 16 c ... at slot c * 8 + (r + c / 2) % 8 -- and are stored as whole 128-byte lines (8 rows x 16 bytes are adjacent
+// in a block).  The loads stay what they are by rows: 16 contiguous bytes per lane.
+template <int CH, bool BLK = false>
+__global__ __launch_bounds__(BLK ? 512 : 256) void act_quant_wave_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
+                                                                         float* __restrict__ xs, int M, int Mp) {
+    constexpr int K = 512 * CH, RPW = BLK ? 8 : 4;
+    __shared__ u32x2 tile[BLK ? CH * 64 * 8 : 1];
+    const int wid = threadIdx.x >> 6, row0 = blockIdx.x * RPW, row = row0 + wid, lane = threadIdx.x & 63;
+    auto gather_store = [&]() {   // BLK: after every wave's codes are in LDS
+        __syncthreads();
+        int8_t* const blk = xq + (size_t(row0 >> 5) * size_t(K >> 5)) * 1024;
+        const u32x4* t16 = reinterpret_cast<const u32x4*>(tile);
+#pragma unroll
+        for (int j = 0; j < CH / 2 + CH % 2; ++j) {   // K / 16 pieces x 8 rows of 16 bytes, 512 per pass
+            const int idx = int(threadIdx.x) + 512 * j, c = idx >> 3, r = idx & 7;
+            if (CH % 2 == 0 || c < K / 16)
+                *reinterpret_cast<u32x4*>(blk + size_t(c >> 1) * 1024 + (c & 1) * 512 + ((row0 + r) & 31) * 16) =
+                    t16[c * 8 + ((r + (c >> 1)) & 7)];
+        }
+    };
+    // piece p (8 codes) of this wave's row: half p % 2 of the 16-byte slot of chunk p / 2
+    auto slot = [&](int p) { return ((p >> 1) * 8 + ((wid + (p >> 2)) & 7)) * 2 + (p & 1); };
+    if (!BLK && row >= Mp) return;
     u32x2* qrow = reinterpret_cast<u32x2*>(xq + size_t(row) * K);
     if (row >= M) {
 #pragma unroll
-        for (int j = 0; j < CH; ++j) qrow[lane + 64 * j] = u32x2{0u, 0u};
+        for (int j = 0; j < CH; ++j) {
+            if (BLK) tile[slot(lane + 64 * j)] = u32x2{0u, 0u}; else qrow[lane + 64 * j] = u32x2{0u, 0u};
+        }
         if (lane == 0) xs[row] = 0.0f;
+        if (BLK) gather_store();
         return;
     }
     const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
@@ -235,31 +257,32 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(const uint16_t* __r
             o[e >> 1] |= (uint32_t(q0) & 0xFFu) << (16 * (e & 1));
             o[e >> 1] |= (uint32_t(q1) & 0xFFu) << (16 * (e & 1) + 8);
         }
-        qrow[lane + 64 * j] = u32x2{o[0], o[1]};
+        if (BLK) tile[slot(lane + 64 * j)] = u32x2{o[0], o[1]}; else qrow[lane + 64 * j] = u32x2{o[0], o[1]};
     }
     if (lane == 0) xs[row] = s;
+    if (BLK) gather_store();
 }
 
 // ---- act_quant into the blocked layout ---------------------------------------------------------------------------
 // xq as the large dense GEMM tiles take it: blocks of 32 rows x 32 k (1 KB), block (m / 32, k / 32) at
 // ((m / 32) * (K / 32) + k / 32) KB, and inside a block the 16 bytes of row r, k half h at (32 h + r) * 16 -- the order
 // in which the 64 lanes of a wave hold a 32x32x32 MFMA operand, so that a wave fetches one block with one coalesced load.
-// One wave per row, eight rows per workgroup.  NJ > 0 (K = 1024 NJ): the row stays in registers (lane l owns the
-// 16-element pieces l, l + 64, ...), and the workgroup's codes meet in LDS, piece by piece, so that they leave as whole
-// 128-byte lines (8 rows x 16 bytes are adjacent in a block).  NJ = 0 (any K % 32 == 0): the row is read twice and every
-// lane writes its own 16 bytes.  Same codes and scales as act_quant_kernel: the row maximum does not depend on the
-// order it is taken in.
-template <int NJ>
+// Rows of K = 512 ... 8192 in steps of 512 go through act_quant_wave_kernel<CH, true> above; this is the kernel for every
+// other K % 32 == 0: one wave per row, eight rows per workgroup, the row read twice, every lane writing the 16 bytes of
+// its own 16 elements.  Same codes and scales as act_quant_kernel: the row maximum does not depend on the order it is
+// taken in.
 __global__ __launch_bounds__(512) void act_quant_blocked_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ xq,
                                                                 float* __restrict__ xs, int M, int Mp, int K) {
-    __shared__ u32x4 tile[NJ > 0 ? NJ * 64 * 8 : 1];   // [piece][row of the workgroup, rotated by piece / 2 over the banks]
-    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = blockIdx.x * 8, row = row0 + w;   // Mp is a multiple of 32: the grid covers whole groups of 8 rows
-    if (NJ > 0) K = 1024 * NJ;
+    const int row = blockIdx.x * 8 + (threadIdx.x >> 6), lane = threadIdx.x & 63;   // Mp % 32 == 0: whole groups of 8 rows
     const int pieces = K / 16;
-    // piece c of a row (k = 16 c ...): k slice c / 2, half c % 2
-    int8_t* const blk = xq + (size_t(row0 >> 5) * size_t(K >> 5)) * 1024;
-    auto at = [&](int c, int r) { return reinterpret_cast<u32x4*>(blk + size_t(c >> 1) * 1024 + (c & 1) * 512 + (r & 31) * 16); };
+    // piece c of the row (k = 16 c ...): k slice c / 2, half c % 2
+    int8_t* const dst = xq + (size_t(row >> 5) * size_t(K >> 5)) * 1024 + size_t(row & 31) * 16;
+    auto at = [&](int c) { return reinterpret_cast<u32x4*>(dst + size_t(c >> 1) * 1024 + (c & 1) * 512); };
+    if (row >= M) {
+        for (int c = lane; c < pieces; c += 64) *at(c) = u32x4{0u, 0u, 0u, 0u};
+        if (lane == 0) xs[row] = 0.0f;
+        return;
+    }
     auto amax8 = [](const u32x4& v, float m) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -280,55 +303,16 @@ __global__ __launch_bounds__(512) void act_quant_blocked_kernel(const uint16_t* 
         return u32x2{o[0], o[1]};
     };
     const u32x4* xrow = reinterpret_cast<const u32x4*>(x + size_t(row) * K);
-    if constexpr (NJ > 0) {
-        u32x4 v[NJ][2];
-        float amax = 0.0f;
-        if (row < M) {
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                v[j][0] = xrow[2 * (lane + 64 * j)];
-                v[j][1] = xrow[2 * (lane + 64 * j) + 1];
-            }
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) amax = amax8(v[j][1], amax8(v[j][0], amax));
-        }
-        amax = wave_max(amax);
-        const float s = __fdiv_rn(amax, 127.0f);
-        const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const int c = lane + 64 * j;
-            u32x4 o = {0u, 0u, 0u, 0u};
-            if (row < M) {
-                const u32x2 lo = codes8(v[j][0], qi), hi = codes8(v[j][1], qi);
-                o = u32x4{lo[0], lo[1], hi[0], hi[1]};
-            }
-            tile[c * 8 + ((w + (c >> 1)) & 7)] = o;
-        }
-        if (lane == 0) xs[row] = row < M ? s : 0.0f;
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {   // 8 consecutive threads carry one 128-byte line: the 8 rows of a piece
-            const int idx = int(threadIdx.x) + 512 * j, c = idx >> 3, r = idx & 7;
-            *at(c, row0 + r) = tile[c * 8 + ((r + (c >> 1)) & 7)];
-        }
-    } else {
-        if (row >= M) {
-            for (int c = lane; c < pieces; c += 64) *at(c, row) = u32x4{0u, 0u, 0u, 0u};
-            if (lane == 0) xs[row] = 0.0f;
-            return;
-        }
-        float amax = 0.0f;
-        for (int c = lane; c < pieces; c += 64) amax = amax8(xrow[2 * c + 1], amax8(xrow[2 * c], amax));
-        amax = wave_max(amax);
-        const float s = __fdiv_rn(amax, 127.0f);
-        const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
-        for (int c = lane; c < pieces; c += 64) {
-            const u32x2 lo = codes8(xrow[2 * c], qi), hi = codes8(xrow[2 * c + 1], qi);
-            *at(c, row) = u32x4{lo[0], lo[1], hi[0], hi[1]};
-        }
-        if (lane == 0) xs[row] = s;
+    float amax = 0.0f;
+    for (int c = lane; c < pieces; c += 64) amax = amax8(xrow[2 * c + 1], amax8(xrow[2 * c], amax));
+    amax = wave_max(amax);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float qi = s > 0.0f ? __fdiv_rn(1.0f, s) : 0.0f;
+    for (int c = lane; c < pieces; c += 64) {
+        const u32x2 lo = codes8(xrow[2 * c], qi), hi = codes8(xrow[2 * c + 1], qi);
+        *at(c) = u32x4{lo[0], lo[1], hi[0], hi[1]};
     }
+    if (lane == 0) xs[row] = s;
 }
 
 // ---- rot_quant: randomized Hadamard rotation of every 32-wide block, then per-token INT8 ---------------------------
@@ -499,14 +483,16 @@ int scmx_act_quant_blocked(const uint16_t* x, int8_t* xq, float* xs, int M, int 
     if (Mp == 0) return SCMX_OK;
     const dim3 grid(unsigned(Mp) / 8u), block(512);
     hipStream_t st = (hipStream_t)stream;
-    switch (K % 1024 ? 0 : K / 1024) {   // rows of up to 8192 elements stay in registers
-        case 1: act_quant_blocked_kernel<1><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
-        case 2: act_quant_blocked_kernel<2><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
-        case 3: act_quant_blocked_kernel<3><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
-        case 4: act_quant_blocked_kernel<4><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
-        case 6: act_quant_blocked_kernel<6><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
-        case 8: act_quant_blocked_kernel<8><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
-        default: act_quant_blocked_kernel<0><<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
+    switch (K % 512 ? 0 : K / 512) {   // rows of up to 8192 elements stay in registers, loaded as by rows
+        case 1: act_quant_wave_kernel<1, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 2: act_quant_wave_kernel<2, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 3: act_quant_wave_kernel<3, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 4: act_quant_wave_kernel<4, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 6: act_quant_wave_kernel<6, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 8: act_quant_wave_kernel<8, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 12: act_quant_wave_kernel<12, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        case 16: act_quant_wave_kernel<16, true><<<grid, block, 0, st>>>(x, xq, xs, M, Mp); break;
+        default: act_quant_blocked_kernel<<<grid, block, 0, st>>>(x, xq, xs, M, Mp, K); break;
     }
     return check_launch("act_quant_blocked");
 }
