@@ -201,7 +201,7 @@ def _rms(x, w, eps, Mp, want_xn, blocked=False):
     _lib.call("scmx_rmsnorm_quant_blocked" if blocked else "scmx_rmsnorm_quant", _lib.ptr(x), _lib.ptr(w), _eps(eps),
               _lib.ptr(xq), _lib.ptr(xs), _lib.ptr(xn), M, Mp, K, _lib.stream())
     if blocked:
-        xq = BlockedXq(xq.reshape(-1), M, K)
+        xq = BlockedXq(xq.reshape(-1), Mp, K)   # Mp rows like the tensor it stands for: the padding rows are zeros
     return (xq, xs, xn) if want_xn else (xq, xs)
 
 
