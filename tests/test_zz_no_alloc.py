@@ -27,8 +27,11 @@ def test_static_scratch_entry_point_equals_the_workspace_one():
     sp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     rng = np.random.default_rng(77)
     # first call large (fills most of a 2048 x 2048 slice of the scratch), second smaller with other K: what the first
-    # call left in the array must not show in the second
-    for (m, n, k, epi) in [(2048, 512, 2048, 1), (300, 384, 1024, 2), (37, 256, 128, 3), (1, 64, 6144, 1)]:
+    # call left in the array must not show in the second.  The 4096-wide case is large enough for the blocked activation
+    # layout (ragged M: the last 32-row block is partly padding); the narrow ones quantize by rows into the same array.
+    shapes = [(2048, 512, 2048, 1), (2047, 4096, 1024, 2), (300, 384, 1024, 2), (37, 256, 128, 3), (1, 64, 6144, 1)]
+    assert lib.scmx_mm_w4a8_prefers_blocked(2047, 4096, 1024) == 1 and lib.scmx_mm_w4a8_prefers_blocked(300, 384, 1024) == 0
+    for (m, n, k, epi) in shapes:
         codes, bc, ws, q = random_packed(rng, n, k)
         bits, x = llm_acts(rng, m, k)
         res = bf16.to_bits(rng.standard_normal((m, n)).astype(F32))
