@@ -244,12 +244,12 @@ def test_swiglu_epilogue_every_gate_value(S):
     assert (~nan).sum() > 2 * 65000
 
 
-def test_linear_layer_replays_in_a_hip_graph(S):
+@pytest.mark.parametrize("n,k,m", [(384, 1024, 200), (4096, 1024, 2047)])   # the second quantizes into the blocked layout
+def test_linear_layer_replays_in_a_hip_graph(S, n, k, m):
     """The entry points only enqueue kernels on the given stream (no allocation, no synchronisation, no memset), so a
     dense layer can be captured once and replayed: every replay, with new activations copied into the captured input
     and eager work in between, equals the eager result bit for bit."""
     rng = np.random.default_rng(21)
-    n, k, m = 384, 1024, 200
     codes, bc, ws, _ = random_packed(rng, n, k)
     dc, db, dw = dev(codes), dev(bc), dev(ws)
     x = torch.zeros((m, k), dtype=torch.bfloat16, device="cuda")
