@@ -1070,6 +1070,10 @@ int scmx_mm_w4a8_blocked(const scmx_format* fmt, const int8_t* xq, const float* 
         set_error("mm_w4a8_blocked: xq must be 16-byte aligned");
         return SCMX_ERR_ARG;
     }
+    if (M > 0 && K > 0 && ((uint64_t(M) + 31) & ~uint64_t(31)) * uint64_t(K) > 0xFFFFFFFFull) {
+        set_error("mm_w4a8_blocked: the activations' whole 32-row blocks lie beyond the 32-bit offsets of the kernel (M=%d K=%d)", M, K);
+        return SCMX_ERR_ARG;
+    }
     return mm_w4a8(fmt, xq, xscale, codes, bcodes, wscale, res, out, epi, M, N, K, true, stream);
 }
 
@@ -1083,7 +1087,8 @@ static int quantize_and_multiply(const scmx_format* fmt, const uint16_t* x, int8
                                  const uint32_t* codes, const uint8_t* bcodes, const float* wscale, const uint16_t* res,
                                  void* out, int epi, int M, int N, int K, void* stream) {
     const long long Mp = (static_cast<long long>(M) + 31) & ~31LL;
-    const bool blocked = room_for_blocks && Mp <= (1LL << 30) && scmx_mm_w4a8_prefers_blocked(M, N, K);
+    const bool blocked = room_for_blocks && Mp <= (1LL << 30) && uint64_t(Mp) * uint64_t(K > 0 ? K : 0) <= 0xFFFFFFFFull &&
+                         scmx_mm_w4a8_prefers_blocked(M, N, K);
     if (blocked) {
         if (int rc = scmx_act_quant_blocked(x, xq, xs, M, int(Mp), K, stream)) return rc;
     } else {
