@@ -237,6 +237,13 @@ def main():
         ops = 2.0 * M_TOKENS * n * k
         per_shape[name] = {"us": round(ms * 1e3, 2), "us_min": round(ms_min * 1e3, 2), "tops": round(ops / ms / 1e9, 1),
                            "pct_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS * 100, 2)}
+        if pre[li][5] and not a.no_sweep:   # the same GEMM on activations quantized by rows, for comparison
+            rq = torch.empty(M_TOKENS * k, dtype=torch.int8, device=dev)
+            check(lib.scmx_act_quant(xs_in[k].data_ptr(), rq.data_ptr(), pre[li][1].data_ptr(), M_TOKENS, M_TOKENS, k, sp))
+            rargs = [(ar[0], rq.data_ptr()) + ar[2:] for _, ar in argl]
+            ms_r, _ = timeit(lambda i: check(lib.scmx_mm_w4a8(*rargs[i % n_sets])), 20, reps=5, warm_s=0.2)
+            per_shape[name]["us_row_layout"] = round(ms_r * 1e3, 2)
+            del rq
         tot_ops += ops
         tot_ms += ms
     achieved = tot_ops / tot_ms / 1e9
